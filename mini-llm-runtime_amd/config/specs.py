@@ -17,13 +17,29 @@ class NormSpec:
     kind: str                 # key in the norm registry, e.g. "rmsnorm"
     size: int
     eps: float
+    weight_offset: float = 0.0    # the factor is weight_offset + the stored weight (1: a weight stored around zero)
+
+
+@dataclass(frozen=True)
+class FrequencyStretch:
+    """Rotation frequencies stretched for contexts beyond the trained one (YaRN): pair i of `dim / 2` pairs lies at
+    d(t) = dim ln(original / (2 pi t)) / (2 ln base) on the scale of turns t over the original length;
+    lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)), dim - 1), ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1);
+    the frequency becomes f_i / factor * ramp_i + f_i (1 - ramp_i), and cosines and sines are multiplied by
+    0.1 ln(factor) + 1."""
+    factor: float
+    original: float
+    fast: float
+    slow: float
 
 
 @dataclass(frozen=True)
 class PositionSpec:
-    kind: str                 # key in the position registry, e.g. "rope_split_half"
+    kind: str                 # key in the position registry: "rope_split_half", or "rope" (which reads every field)
     dim: int                  # rotated width (the head size here)
     base: float
+    interleaved: bool = False                      # pairs (2 i, 2 i + 1) instead of (i, i + dim / 2)
+    stretch: Optional[FrequencyStretch] = None
 
 
 @dataclass(frozen=True)
@@ -44,7 +60,7 @@ class MlpSpec:
     kind: str                 # key in the feed-forward registry, e.g. "swiglu"
     hidden: int
     intermediate: int
-    activation: str = "silu"
+    activation: str = "silu"  # of the gate: silu, gelu_tanh
 
 
 @dataclass(frozen=True)
@@ -139,6 +155,9 @@ class SinkAttentionSpec:
     mask: Optional[MaskSpec] = None              # None: every earlier key
     sink: bool = True
     bias: bool = False
+    qk_norm_weight: bool = True                  # False: q and k are only divided by their root mean square
+    qk_norm_after_rotation: bool = False         # the norm follows the rotation instead of preceding it
+    gate: Optional[str] = None                   # "sigmoid": the heads side by side times sigmoid(Wg x) before Wo
 
 
 @dataclass(frozen=True)
@@ -159,6 +178,52 @@ class LatentAttentionSpec:
     position: PositionSpec = None                # turns the whole rotated part: dim == rot_dim
     mask: Optional[MaskSpec] = None
     sink: bool = True
+    q_rank: Optional[int] = None                 # queries through a normed latent of their own: Wuq norm(Wdq x)
+
+
+@dataclass(frozen=True)
+class DecayedLinearAttentionSpec:
+    """Linear attention with ONE constant decay a head: q, k, v = act(W x); per head S_t = decay S_(t-1) + k_t v_t^T,
+    o_t = S_t^T q_t; the heads side by side are RMS-normed as one row (a weight as wide as the row), multiplied by
+    gate(Wg x) and projected by Wo."""
+    kind: str                 # "decayed_linear_attention"
+    hidden: int
+    heads: int
+    head_dim: int
+    value_dim: int
+    decay: Tuple[float, ...]  # one number in (0, 1] a head
+    eps: float
+    activation: str = "silu"
+    gate: str = "sigmoid"
+
+
+@dataclass(frozen=True)
+class DeltaRuleSpec:
+    """Gated delta rule with a decay per key channel: q, k (kv_heads x head_dim) and v (heads x value_dim) pass a short
+    causal convolution and silu; q and k are made unit vectors per head (x / sqrt(sum x^2 + unit_eps)), q times
+    head_dim^(-1/2); beta = sigmoid(Wb x) a head; g = exp(-exp(A_log[head]) softplus(Wa2 (Wa1 x) + dt_bias)) per head
+    and key channel; per head S <- diag(g) S, u = beta (v - S^T k), S <- S + k u^T, o = S^T q; each head's o over its
+    root mean square, times a weight shared by the heads, times sigmoid(Wg2 (Wg1 x)); then Wo."""
+    kind: str                 # "delta_rule"
+    hidden: int
+    heads: int
+    kv_heads: int
+    head_dim: int
+    value_dim: int
+    conv_taps: int
+    eps: float
+    unit_eps: float = 1e-6
+    decay_rank: Optional[int] = None      # None: the file's tensors say
+    gate_rank: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class MixerSumSpec:
+    """Several mixers side by side on the same input: the output is sum_i scale_i mixer_i(x).  `mixers`: (name, spec,
+    scale) each; a mixer's tensors are named `<name>.<its local name>`, and each keeps a cache entry of its own."""
+    kind: str                 # "mixer_sum"
+    hidden: int
+    mixers: Tuple[Tuple[str, object, float], ...]
 
 
 @dataclass(frozen=True)
@@ -211,6 +276,18 @@ class EmbedSpec:
     kind: str                 # key in the embed registry, e.g. "token_embedding"
     vocab_size: int
     hidden: int
+
+
+@dataclass(frozen=True)
+class PairEmbedSpec:
+    """A token's embedding plus a row of a second table picked by the token and the one before it:
+    row (previous * mul_prev + token * mul_cur) mod buckets, and row number `buckets` for a sequence's first token."""
+    kind: str                 # "pair_embedding"
+    vocab_size: int
+    hidden: int
+    buckets: int
+    mul_prev: int
+    mul_cur: int
 
 
 @dataclass(frozen=True)

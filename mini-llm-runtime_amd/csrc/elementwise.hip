@@ -238,7 +238,16 @@ __global__ void residual_add_kernel(float* __restrict__ h, const elem_t* __restr
     }
 }
 
+// The activation of a gated feed-forward's gate: ACT 0 silu(g) = g / (1 + exp(-g)); ACT 1 the tanh form of gelu,
+// 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))).  32-bit.
+template <int ACT>
+__device__ __forceinline__ float gate_act(float g) {
+    if (ACT == 1) return 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+    return g / (1.0f + expf(-g));
+}
+
 // The same, 16 bytes per lane and access, for inter % MLR_VEC == 0.
+template <int ACT>
 __global__ void silu_mul_vec_kernel(const elem_t* __restrict__ gate_up, elem_t* __restrict__ act, int rows, int inter) {
     const int per_row = inter / MLR_VEC;
     const size_t total = (size_t)rows * per_row;
@@ -248,12 +257,13 @@ __global__ void silu_mul_vec_kernel(const elem_t* __restrict__ gate_up, elem_t* 
         load_vec(gate_up + m * 2 * inter + f, g);
         load_vec(gate_up + m * 2 * inter + inter + f, u);
 #pragma unroll
-        for (int e = 0; e < MLR_VEC; ++e) y[e] = (g[e] / (1.0f + expf(-g[e]))) * u[e];
+        for (int e = 0; e < MLR_VEC; ++e) y[e] = gate_act<ACT>(g[e]) * u[e];
         store_vec(act + m * inter + f, y);
     }
 }
 
-// act[m, f] = silu(gate_up[m, f]) * gate_up[m, inter + f]; silu(g) = g / (1 + exp(-g)).
+// act[m, f] = act(gate_up[m, f]) * gate_up[m, inter + f].
+template <int ACT>
 __global__ void silu_mul_kernel(const elem_t* __restrict__ gate_up, elem_t* __restrict__ act,
                                 int rows, int inter) {
     const size_t total = (size_t)rows * inter;
@@ -262,8 +272,76 @@ __global__ void silu_mul_kernel(const elem_t* __restrict__ gate_up, elem_t* __re
         const size_t m = i / inter, f = i % inter;
         const float g = to_float(gate_up[m * 2 * inter + f]);
         const float u = to_float(gate_up[m * 2 * inter + inter + f]);
-        act[i] = from_float<elem_t>((g / (1.0f + expf(-g))) * u);
+        act[i] = from_float<elem_t>(gate_act<ACT>(g) * u);
     }
+}
+
+// The embedding of a token plus the row of a pair table that the token and the one before it pick:
+// h[m] = float(table[id]) + float(pairs[row]), row = (previous * mul_prev + id * mul_cur) mod buckets, and the table's
+// last row (number `buckets`) for a request's first token (position 0).  The token before row m is the row above it
+// when that row is the same request's previous position, else what the request's state holds (`live[slot]`); the
+// last row that a request brings to the step leaves its token in `stage[slot]`.  An id outside [0, vocab) gives a
+// row of NaN (the host refuses such a batch before anything runs).
+__global__ void pair_embed_kernel(const int32_t* __restrict__ ids, const int32_t* __restrict__ positions,
+                                  const int32_t* __restrict__ slots, const elem_t* __restrict__ table,
+                                  const elem_t* __restrict__ pairs, const int32_t* __restrict__ live,
+                                  int32_t* __restrict__ stage, float* __restrict__ h, int rows, int width, int vocab,
+                                  int buckets, long long mul_prev, long long mul_cur) {
+    const int m = blockIdx.x;
+    const int id = ids[m], pos = positions[m], slot = slots[m];
+    float* out = h + (size_t)m * width;
+    const bool last = m + 1 >= rows || slots[m + 1] != slot || positions[m + 1] != pos + 1;
+    if (last && threadIdx.x == 0) stage[slot] = id;
+    if (id < 0 || id >= vocab) {
+        for (int i = threadIdx.x; i < width; i += blockDim.x) out[i] = __int_as_float(0x7fc00000);
+        return;
+    }
+    long long pair = buckets;
+    if (pos > 0) {
+        const int before = m > 0 && slots[m - 1] == slot && positions[m - 1] == pos - 1 ? ids[m - 1] : live[slot];
+        pair = ((long long)before * mul_prev + (long long)id * mul_cur) % buckets;
+        if (pair < 0) pair += buckets;
+    }
+    const elem_t* row = table + (size_t)id * width;
+    const elem_t* add = pairs + (size_t)pair * width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) out[i] = to_float(row[i]) + to_float(add[i]);
+}
+
+// out[m, c] = scale * x[m, c] * act(gate[m * gate_stride + c]); ACT 0 silu, 1 sigmoid.  32-bit inside.
+template <int ACT>
+__global__ void gate_mul_kernel(const elem_t* __restrict__ x, const elem_t* __restrict__ gate, long gate_stride,
+                                elem_t* __restrict__ out, size_t rows, int width, float scale) {
+    const size_t total = rows * width;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t m = i / width, c = i % width;
+        const float g = to_float(gate[m * gate_stride + c]);
+        const float s = 1.0f / (1.0f + expf(-g));
+        out[i] = from_float<elem_t>(scale * (to_float(x[i]) * (ACT == 0 ? g * s : s)));
+    }
+}
+
+// out[m] = x[m] / sqrt(mean(x[m]^2) + eps) * weight for a block of columns x[m * x_stride + c] of a wider matrix
+// (a latent vector that comes out of a projection beside other things); 32-bit inside.  One workgroup a row.
+__global__ __launch_bounds__(256) void rmsnorm_columns_kernel(const elem_t* __restrict__ x, long x_stride,
+                                                              const float* __restrict__ weight, elem_t* __restrict__ out,
+                                                              int width, float eps) {
+    __shared__ float scratch[16];
+    const elem_t* row = x + (size_t)blockIdx.x * x_stride;
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float v = to_float(row[i]);
+        sum += v * v;
+    }
+    const float r = 1.0f / sqrtf(block_sum(sum, scratch) / (float)width + eps);
+    for (int i = threadIdx.x; i < width; i += blockDim.x)
+        out[(size_t)blockIdx.x * width + i] = from_float<elem_t>((to_float(row[i]) * r) * weight[i]);
+}
+
+// out = sa * a + sb * b, the sum taken in 32-bit.
+__global__ void scaled_sum_kernel(const elem_t* __restrict__ a, const elem_t* __restrict__ b, elem_t* __restrict__ out,
+                                  float sa, float sb, size_t count) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+        out[i] = from_float<elem_t>(sa * to_float(a[i]) + sb * to_float(b[i]));
 }
 
 // The first half of an RMSNorm whose scale is applied by the projection that follows (few rows): x = h + delta
@@ -644,6 +722,18 @@ static int grid_for(size_t count, int block) {
     return (int)(g > 65535 ? 65535 : (g == 0 ? 1 : g));
 }
 
+template <int ACT>
+static int launch_gated(const void* gate_up, void* act, int rows, int inter, hipStream_t stream) {
+    if (inter % MLR_VEC == 0) {
+        silu_mul_vec_kernel<ACT><<<grid_for((size_t)rows * (inter / MLR_VEC), 256), 256, 0, stream>>>(
+            (const elem_t*)gate_up, (elem_t*)act, rows, inter);
+        return (int)hipGetLastError();
+    }
+    silu_mul_kernel<ACT><<<grid_for((size_t)rows * inter, 256), 256, 0, stream>>>(
+        (const elem_t*)gate_up, (elem_t*)act, rows, inter);
+    return (int)hipGetLastError();
+}
+
 extern "C" {
 
 int mlr_embed_gather(const int32_t* ids, const void* table, float* h, int rows, int width, int vocab,
@@ -700,13 +790,53 @@ int mlr_residual_add(float* h, const void* delta, size_t count, hipStream_t stre
 
 int mlr_silu_mul(const void* gate_up, void* act, int rows, int inter, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (inter % MLR_VEC == 0) {
-        silu_mul_vec_kernel<<<grid_for((size_t)rows * (inter / MLR_VEC), 256), 256, 0, stream>>>(
-            (const elem_t*)gate_up, (elem_t*)act, rows, inter);
-        return (int)hipGetLastError();
-    }
-    silu_mul_kernel<<<grid_for((size_t)rows * inter, 256), 256, 0, stream>>>(
-        (const elem_t*)gate_up, (elem_t*)act, rows, inter);
+    return launch_gated<0>(gate_up, act, rows, inter, stream);
+}
+
+// act = activation(gate) * up; kind 0: silu, 1: the tanh form of gelu
+int mlr_gated_act_mul(const void* gate_up, void* act, int rows, int inter, int kind, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (kind == 0) return launch_gated<0>(gate_up, act, rows, inter, stream);
+    if (kind == 1) return launch_gated<1>(gate_up, act, rows, inter, stream);
+    return -1;
+}
+
+int mlr_pair_embed(const int32_t* ids, const int32_t* positions, const int32_t* slots, const void* table, const void* pairs,
+                   const int32_t* live, int32_t* stage, float* h, int rows, int width, int vocab, int buckets,
+                   long long mul_prev, long long mul_cur, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (buckets < 1) return -1;
+    pair_embed_kernel<<<rows, 256, 0, stream>>>(ids, positions, slots, (const elem_t*)table, (const elem_t*)pairs, live, stage,
+                                                h, rows, width, vocab, buckets, mul_prev, mul_cur);
+    return (int)hipGetLastError();
+}
+
+// out = scale * x * act(gate); kind 0: silu, 1: sigmoid; gate: columns of a row-major matrix
+int mlr_gate_mul(const void* x, const void* gate, long gate_stride, void* out, int rows, int width, int kind, float scale,
+                 hipStream_t stream) {
+    if (rows <= 0 || width <= 0) return 0;
+    const int grid = grid_for((size_t)rows * width, 256);
+    if (kind == 0)
+        gate_mul_kernel<0><<<grid, 256, 0, stream>>>((const elem_t*)x, (const elem_t*)gate, gate_stride, (elem_t*)out,
+                                                     (size_t)rows, width, scale);
+    else if (kind == 1)
+        gate_mul_kernel<1><<<grid, 256, 0, stream>>>((const elem_t*)x, (const elem_t*)gate, gate_stride, (elem_t*)out,
+                                                     (size_t)rows, width, scale);
+    else
+        return -1;
+    return (int)hipGetLastError();
+}
+
+int mlr_rmsnorm_columns(const void* x, long x_stride, const float* weight, void* out, int rows, int width, float eps,
+                        hipStream_t stream) {
+    if (rows <= 0 || width <= 0) return 0;
+    rmsnorm_columns_kernel<<<rows, 256, 0, stream>>>((const elem_t*)x, x_stride, weight, (elem_t*)out, width, eps);
+    return (int)hipGetLastError();
+}
+
+int mlr_scaled_sum(const void* a, const void* b, void* out, float sa, float sb, size_t count, hipStream_t stream) {
+    if (count == 0) return 0;
+    scaled_sum_kernel<<<grid_for(count, 256), 256, 0, stream>>>((const elem_t*)a, (const elem_t*)b, (elem_t*)out, sa, sb, count);
     return (int)hipGetLastError();
 }
 

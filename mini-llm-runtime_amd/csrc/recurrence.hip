@@ -8,6 +8,9 @@
 // layer has run).  Every sum is taken in an order that depends on the token's own data only, so a token's
 // result does not depend on how its request was cut into steps or on what else the batch holds.
 //
+// The delta rule (`delta_rule_kernel`) is the same walk with a write that first takes back what the state already
+// holds for the token's key:  S <- diag(g_t) S;  u = beta_t (v_t - S^T k_t);  S <- S + k_t u^T;  o_t = S^T q_t.
+//
 // Long portions (the bfloat16 engine) run the recurrence over pieces of a request side by side, in three passes:
 // every piece from a zero state, leaving its last state L_c and the product A_c of its decays; then, piece after
 // piece, the state each piece starts from, S_(c+1) = diag(A_c) S_c + L_c (element by element, from the live
@@ -16,6 +19,8 @@
 #include "common.h"
 
 __device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
+__device__ __forceinline__ float silu_f(float x) { return x / (1.0f + expf(-x)); }
+__device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 
 // ---- short causal convolution -----------------------------------------------------------------------
 // out[r, c] = act(b[c] + sum_j w[c, j] * in(r, taps - 1 - j)) with in(r, d) the channel's input d tokens before
@@ -102,6 +107,7 @@ struct ScanArgs {
     const int32_t* seg_first; const int32_t* seg_count; const int32_t* slots;
     int heads, heads_per_group, N, V, decay_per_channel, write_state;
     float q_scale;
+    int silu;                                  // q, k and v pass silu as they are read (before the factors)
     float* piece_state;                        // [pieces][heads][N][V]: L_c after the first pass, S_c after the second
     float* piece_decay;                        // [pieces][heads][N]: A_c
 };
@@ -152,7 +158,9 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(ScanArgs a) {
             if (i < N) {
                 da = expf(a.log_decay[row * a.decay_stride + (a.decay_per_channel ? head * N + i : head)]);
                 dk = to_float(a.k[row * a.k_stride + qk_head * N + i]);
-                dq = to_float(a.q[row * a.q_stride + qk_head * N + i]) * a.q_scale;
+                dq = to_float(a.q[row * a.q_stride + qk_head * N + i]);
+                if (a.silu) { dk = silu_f(dk); dq = silu_f(dq); }
+                dq *= a.q_scale;
             }
             a_lds[idx] = da; k_lds[idx] = dk; q_lds[idx] = dq;
         }
@@ -162,6 +170,7 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(ScanArgs a) {
             float x = 0.f;
             if (c < V) {
                 x = to_float(a.v[row * a.v_stride + head * V + c]);
+                if (a.silu) x = silu_f(x);
                 if (a.v_scale) x *= a.v_scale[row * a.v_scale_stride + head];
             }
             v_lds[idx] = x;
@@ -190,7 +199,10 @@ __global__ __launch_bounds__(256) void linear_recurrence_kernel(ScanArgs a) {
             float o = o_lds[idx];
 #pragma unroll
             for (int p = 1; p < SCAN_PARTS; ++p) o += o_lds[p * TILE * SCAN_COLS + idx];
-            if (a.skip) o += a.skip[head] * to_float(a.v[row * a.v_stride + head * V + c]);
+            if (a.skip) {
+                const float x = to_float(a.v[row * a.v_stride + head * V + c]);
+                o += a.skip[head] * (a.silu ? silu_f(x) : x);
+            }
             a.out[row * ((size_t)a.heads * V) + head * V + c] = o;
         }
     }
@@ -228,6 +240,140 @@ __global__ void piece_states_kernel(ScanArgs a, int pieces) {
         S = a.piece_decay[(size_t)c * a.heads * a.N + hi] * S + last;
         if (a.write_state && (c + 1 == pieces || a.slots[a.seg_first[c + 1]] != slot)) a.stage[(size_t)slot * a.state_stride + e] = S;
     }
+}
+
+// ---- the delta rule ----------------------------------------------------------------------------------------
+// Decays of the key channels from a step size per channel: log g = -exp(A_log[head]) * softplus(z + bias), z the
+// 32-bit output of a low-rank pair of projections laid out [heads][N].
+__global__ void channel_log_decay_kernel(const float* __restrict__ z, const float* __restrict__ bias,
+                                         const float* __restrict__ a_log, float* __restrict__ out, size_t rows, int width,
+                                         int per_head) {
+    const size_t total = rows * width;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const int c = (int)(i % width);
+        out[i] = -expf(a_log[c / per_head]) * softplus_f(z[i] + (bias ? bias[c] : 0.f));
+    }
+}
+
+struct DeltaArgs {
+    const elem_t* q; long q_stride;            // q[r * q_stride + (head / heads_per_group) * N + i], as projected
+    const elem_t* k; long k_stride;
+    const elem_t* v; long v_stride;            // v[r * v_stride + head * V + j]
+    const float* log_decay;                    // [rows][heads * N]
+    const float* beta_raw; long beta_stride;   // beta = sigmoid(beta_raw[r * stride + head])
+    float* out;                                // [rows, heads * V]
+    const float* live; float* stage; long state_stride;     // a request's S as [heads][N][V]
+    const int32_t* seg_first; const int32_t* seg_count; const int32_t* slots;
+    int heads, heads_per_group, N, V, write_state, unit_norm;
+    float q_scale, unit_eps;
+};
+
+#define DELTA_TILE 16
+
+// One wavefront per (request of the step, head, COLS value channels), COLS = 64 / PARTS: lane (part, column) holds
+// rows [part NR, (part + 1) NR) of its column of S in registers.  Tokens are staged DELTA_TILE at a time through LDS:
+// q and k made unit vectors over the head's N channels (x / sqrt(sum x^2 + unit_eps); q times q_scale), the decays
+// exponentiated, beta = sigmoid(raw), k . q of every token.  A token then costs one pass over the lane's rows for
+// (g S)^T k and (g S)^T q, an exchange between the parts, and one pass for the write; the read-out after the write is
+// o = (g S)^T q + (k . q) u.  Every sum's order follows from the head's sizes alone.
+template <int NR, int PARTS>
+__global__ __launch_bounds__(64) void delta_rule_kernel(DeltaArgs a) {
+    constexpr int COLS = 64 / PARTS;
+    constexpr int NPAD = NR * PARTS;
+    __shared__ __attribute__((aligned(16))) float g_lds[DELTA_TILE * NPAD];
+    __shared__ __attribute__((aligned(16))) float k_lds[DELTA_TILE * NPAD];
+    __shared__ __attribute__((aligned(16))) float q_lds[DELTA_TILE * NPAD];
+    __shared__ float v_lds[DELTA_TILE * COLS];
+    __shared__ float beta_lds[DELTA_TILE], kq_lds[DELTA_TILE];
+    const int seg = blockIdx.x, head = blockIdx.y, col0 = blockIdx.z * COLS;
+    const int r0 = a.seg_first[seg], n = a.seg_count[seg];
+    const int slot = a.slots[r0];
+    const int lane = threadIdx.x, j = lane % COLS, part = lane / COLS;
+    const int col = col0 + j;
+    const int N = a.N, V = a.V;
+    const int qk_head = head / a.heads_per_group;
+    const size_t state_at = (size_t)slot * a.state_stride + (size_t)head * N * V;
+    float S[NR];
+#pragma unroll
+    for (int r = 0; r < NR; ++r) {
+        const int i = part * NR + r;
+        S[r] = i < N && col < V ? a.live[state_at + (size_t)i * V + col] : 0.f;
+    }
+    for (int t0 = 0; t0 < n; t0 += DELTA_TILE) {
+        const int nt = min(DELTA_TILE, n - t0);
+        __syncthreads();                                  // the tile before has been read
+        for (int t = 0; t < nt; ++t) {
+            const size_t row = (size_t)(r0 + t0 + t);
+            float qq = 0.f, kk = 0.f;
+            for (int i = lane; i < NPAD; i += 64) {
+                float dq = 0.f, dk = 0.f, dg = 0.f;
+                if (i < N) {
+                    dq = to_float(a.q[row * a.q_stride + qk_head * N + i]);
+                    dk = to_float(a.k[row * a.k_stride + qk_head * N + i]);
+                    dg = expf(a.log_decay[row * ((size_t)a.heads * N) + head * N + i]);
+                }
+                qq += dq * dq;
+                kk += dk * dk;
+                q_lds[t * NPAD + i] = dq; k_lds[t * NPAD + i] = dk; g_lds[t * NPAD + i] = dg;
+            }
+            float fq = a.q_scale, fk = 1.0f;
+            if (a.unit_norm) {
+                fq = a.q_scale / sqrtf(wave_sum(qq) + a.unit_eps);
+                fk = 1.0f / sqrtf(wave_sum(kk) + a.unit_eps);
+            }
+            float dot = 0.f;
+            for (int i = lane; i < NPAD; i += 64) {      // (each lane returns to the channels it wrote)
+                const float dq = q_lds[t * NPAD + i] * fq, dk = k_lds[t * NPAD + i] * fk;
+                q_lds[t * NPAD + i] = dq; k_lds[t * NPAD + i] = dk;
+                dot += dq * dk;
+            }
+            dot = wave_sum(dot);
+            if (lane == 0) {
+                kq_lds[t] = dot;
+                beta_lds[t] = sigmoid_f(a.beta_raw[row * a.beta_stride + head]);
+            }
+        }
+        for (int idx = lane; idx < nt * COLS; idx += 64) {
+            const int t = idx / COLS, c = col0 + idx % COLS;
+            v_lds[idx] = c < V ? to_float(a.v[(size_t)(r0 + t0 + t) * a.v_stride + head * V + c]) : 0.f;
+        }
+        __syncthreads();
+        for (int t = 0; t < nt; ++t) {
+            const float* gt = g_lds + t * NPAD + part * NR;
+            const float* kt = k_lds + t * NPAD + part * NR;
+            const float* qt = q_lds + t * NPAD + part * NR;
+            float sk = 0.f, sq = 0.f;
+#pragma unroll
+            for (int r = 0; r < NR; ++r) {
+                S[r] *= gt[r];
+                sk += kt[r] * S[r];
+                sq += qt[r] * S[r];
+            }
+#pragma unroll
+            for (int off = COLS; off < 64; off <<= 1) {   // the parts of a column lie COLS lanes apart
+                sk += __shfl_xor(sk, off, 64);
+                sq += __shfl_xor(sq, off, 64);
+            }
+            const float u = beta_lds[t] * (v_lds[t * COLS + j] - sk);
+#pragma unroll
+            for (int r = 0; r < NR; ++r) S[r] += kt[r] * u;
+            if (part == 0 && col < V) a.out[(size_t)(r0 + t0 + t) * ((size_t)a.heads * V) + head * V + col] = sq + kq_lds[t] * u;
+        }
+    }
+    if (a.write_state && col < V) {
+#pragma unroll
+        for (int r = 0; r < NR; ++r) {
+            const int i = part * NR + r;
+            if (i < N) a.stage[state_at + (size_t)i * V + col] = S[r];
+        }
+    }
+}
+
+template <int NR, int PARTS>
+static int launch_delta(const DeltaArgs& a, int segments, hipStream_t stream) {
+    constexpr int COLS = 64 / PARTS;
+    delta_rule_kernel<NR, PARTS><<<dim3(segments, a.heads, (a.V + COLS - 1) / COLS), 64, 0, stream>>>(a);
+    return (int)hipGetLastError();
 }
 
 template <int NR, int TILE>
@@ -287,20 +433,62 @@ int mlr_linear_recurrence(const void* q, long q_stride, const void* k, long k_st
                           long v_scale_stride, const float* skip, float q_scale, float* out, const float* live, float* stage,
                           long state_stride, const int32_t* seg_first, const int32_t* seg_count, const int32_t* slots,
                           int segments, int heads, int heads_per_group, int n_keys, int n_values, int write_state,
-                          float* piece_state, float* piece_decay, hipStream_t stream) {
+                          float* piece_state, float* piece_decay, int silu, hipStream_t stream) {
     // piece_state, piece_decay given: `seg_first`/`seg_count` name pieces of requests (a request's pieces one after
     // the other), run side by side in three passes; [segments][heads][n_keys][n_values] and [segments][heads][n_keys]
     if (segments <= 0) return 0;
     if (n_keys < 1 || n_keys > 256 || n_values < 1 || heads < 1 || heads_per_group < 1 || heads % heads_per_group) return -1;
     ScanArgs a{(const elem_t*)q, q_stride, (const elem_t*)k, k_stride, (const elem_t*)v, v_stride, log_decay, decay_stride,
                v_scale, v_scale_stride, skip, out, live, stage, state_stride, seg_first, seg_count, slots, heads,
-               heads_per_group, n_keys, n_values, decay_per_channel, write_state, q_scale, piece_state, piece_decay};
+               heads_per_group, n_keys, n_values, decay_per_channel, write_state, q_scale, silu, piece_state, piece_decay};
     if ((piece_state == nullptr) != (piece_decay == nullptr)) return -2;
     const int nr = (n_keys + SCAN_PARTS - 1) / SCAN_PARTS;
     if (nr <= 8) return launch_scan<8, 16>(a, segments, stream);
     if (nr <= 16) return launch_scan<16, 16>(a, segments, stream);
     if (nr <= 32) return launch_scan<32, 16>(a, segments, stream);
     return launch_scan<64, 8>(a, segments, stream);
+}
+
+int mlr_channel_log_decay(const float* z, const float* bias, const float* a_log, float* out, int rows, int heads, int n_keys,
+                          hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (heads < 1 || n_keys < 1) return -1;
+    channel_log_decay_kernel<<<grid_for((size_t)rows * heads * n_keys, 256), 256, 0, stream>>>(z, bias, a_log, out, (size_t)rows,
+                                                                                            heads * n_keys, n_keys);
+    return (int)hipGetLastError();
+}
+
+// The delta rule over the step's requests (seg_first, seg_count: one entry a request).  A lane keeps at most 64 rows of
+// its column of S: up to 64 key channels a lane holds a whole column (64 columns a wavefront), up to 128 two lanes share
+// one, up to 256 four; heads of few value channels use the narrower layouts too, so that their lanes are not idle.
+int mlr_delta_rule(const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
+                   const float* log_decay, const float* beta_raw, long beta_stride, float* out, const float* live, float* stage,
+                   long state_stride, const int32_t* seg_first, const int32_t* seg_count, const int32_t* slots, int segments,
+                   int heads, int heads_per_group, int n_keys, int n_values, int write_state, int unit_norm, float q_scale,
+                   float unit_eps, hipStream_t stream) {
+    if (segments <= 0) return 0;
+    if (n_keys < 1 || n_keys > 256 || n_values < 1 || heads < 1 || heads > 65535 || heads_per_group < 1 ||
+        heads % heads_per_group)
+        return -1;
+    DeltaArgs a{(const elem_t*)q, q_stride, (const elem_t*)k, k_stride, (const elem_t*)v, v_stride, log_decay, beta_raw,
+                beta_stride, out, live, stage, state_stride, seg_first, seg_count, slots, heads, heads_per_group, n_keys,
+                n_values, write_state, unit_norm, q_scale, unit_eps};
+    int parts = n_keys > 128 ? 4 : n_keys > 64 ? 2 : 1;
+    if (n_values <= 16 && parts < 4) parts = 4;
+    else if (n_values <= 32 && parts < 2) parts = 2;
+    const int nr = (n_keys + parts - 1) / parts;
+#define MLR_DELTA(PARTS)                                                        \
+    if (parts == PARTS) {                                                       \
+        if (nr <= 8) return launch_delta<8, PARTS>(a, segments, stream);        \
+        if (nr <= 16) return launch_delta<16, PARTS>(a, segments, stream);      \
+        if (nr <= 32) return launch_delta<32, PARTS>(a, segments, stream);      \
+        return launch_delta<64, PARTS>(a, segments, stream);                    \
+    }
+    MLR_DELTA(1)
+    MLR_DELTA(2)
+    MLR_DELTA(4)
+#undef MLR_DELTA
+    return -1;
 }
 
 }  // extern "C"

@@ -138,17 +138,31 @@ __global__ __launch_bounds__(64) void sink_attention_kernel(SinkArgs a) {
 // ---------------------------------------------------------------------------------------------------------
 // Queries, keys and values of a grouped-query attention from the stacked projection's output
 // proj[m] = [q_heads * key_dim | kv_heads * key_dim | kv_heads * value_dim]: the projection's bias added (null:
-// none), q and k normed per head over key_dim (x / sqrt(mean(x^2) + eps) * weight, the weight shared by the
-// heads; null: no norm), the first rot_dim channels of a head turned by the token's position in pairs
-// (j, j + rot_dim / 2) with cos = table[p][j], sin = table[p][rot_dim / 2 + j] (table null: no rotation);
+// none); q and k normed per head over key_dim (x / sqrt(mean(x^2) + eps) * weight, the weight shared by the
+// heads; null: no weight) before the rotation (norm_mode 1), after it (norm_mode 2) or not at all (0); the first
+// rot_dim channels of a head turned by the token's position with cos = table[p][j], sin = table[p][rot_dim / 2 + j]
+// in pairs (j, j + rot_dim / 2) or, `interleaved`, (2 j, 2 j + 1) (table null: no rotation);
 // q to q_out [m, q_heads * key_dim], k and v into their pages.  One wavefront a head; 32-bit throughout.
+__device__ __forceinline__ float turned_channel(const float* x, int d, const float* cs, int rot_dim, int interleaved) {
+    if (cs == nullptr || d >= rot_dim) return x[d];
+    const int half = rot_dim >> 1;
+    if (interleaved) {
+        const int j = d >> 1;
+        const float c = cs[j], s = cs[half + j];
+        return (d & 1) ? turn_y(x[d - 1], x[d], c, s) : turn_x(x[d], x[d + 1], c, s);
+    }
+    const int j = d < half ? d : d - half;
+    const float c = cs[j], s = cs[half + j];
+    return d < half ? turn_x(x[d], x[d + half], c, s) : turn_y(x[d - half], x[d], c, s);
+}
+
 __global__ __launch_bounds__(64) void sink_qkv_prep_kernel(
     const elem_t* __restrict__ proj, long ld, const float* __restrict__ bias, elem_t* __restrict__ q_out,
     elem_t* __restrict__ k_pages, long k_row, elem_t* __restrict__ v_pages, long v_row,
     const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ slots,
     const int32_t* __restrict__ positions, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
     float eps, const float* __restrict__ rope, int rot_dim, int q_heads, int kv_heads, int key_dim, int value_dim,
-    int page_size, int write_cache) {
+    int page_size, int write_cache, int norm_mode, int interleaved) {
     __shared__ float x_lds[MAX_KEY_DIM];
     const int m = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
     const int pos = positions[m], slot = slots[m];
@@ -176,50 +190,60 @@ __global__ __launch_bounds__(64) void sink_qkv_prep_kernel(
         x_lds[d] = x;
         sum += x * x;
     }
-    if (w != nullptr) {
+    if (norm_mode == 1) {
         sum = wave_sum(sum);
         const float r = 1.0f / sqrtf(sum / (float)key_dim + eps);
-        for (int d = lane; d < key_dim; d += 64) x_lds[d] = (x_lds[d] * r) * w[d];
+        for (int d = lane; d < key_dim; d += 64) x_lds[d] = (x_lds[d] * r) * (w != nullptr ? w[d] : 1.0f);
     }
     __syncthreads();
     elem_t* dst = unit < q_heads ? q_out + ((size_t)m * q_heads + unit) * key_dim : k_pages + cache_row * k_row;
-    const int half = rot_dim >> 1;
     const float* cs = rope ? rope + (size_t)pos * rot_dim : nullptr;
-    for (int d = lane; d < key_dim; d += 64) {
-        float y = x_lds[d];
-        if (cs != nullptr && d < rot_dim) {
-            const int j = d < half ? d : d - half;
-            const float c = cs[j], s = cs[half + j];
-            y = d < half ? turn_x(x_lds[d], x_lds[d + half], c, s) : turn_y(x_lds[d - half], x_lds[d], c, s);
+    float r_after = 1.0f;
+    if (norm_mode == 2) {                       // the root mean square of the head as it is after the rotation
+        float turned = 0.f;
+        for (int d = lane; d < key_dim; d += 64) {
+            const float y = turned_channel(x_lds, d, cs, rot_dim, interleaved);
+            turned += y * y;
         }
+        turned = wave_sum(turned);
+        r_after = 1.0f / sqrtf(turned / (float)key_dim + eps);
+    }
+    for (int d = lane; d < key_dim; d += 64) {
+        float y = turned_channel(x_lds, d, cs, rot_dim, interleaved);
+        if (norm_mode == 2) y = (y * r_after) * (w != nullptr ? w[d] : 1.0f);
         dst[d] = from_float<elem_t>(y);
     }
 }
 
-// Latent attention's row work.  proj[m] = [heads * (dim + rot) | rank + rot]: per head `dim` plain and `rot`
-// rotated query channels, then the latent part (`rank` channels) and the one rotated key part all heads share.
+// Latent attention's row work.  q_src[m] = [heads * (dim + rot)]: per head `dim` plain and `rot` rotated query
+// channels; kv_src[m] = [rank + rot]: the latent part (`rank` channels) and the one rotated key part all heads
+// share (the two may be column blocks of one projection's output).
 //   units 0 .. heads - 1: the head's rotated query channels, turned by the token's position (pairs
-//     (j, j + rot / 2)), to q_out[m][head][rank .. rank + rot) -- the plain channels reach
-//     q_out[m][head][0 .. rank) through the key up-projection, which is another kernel's work;
+//     (j, j + rot / 2) or, `interleaved`, (2 j, 2 j + 1)), to q_out[m][head][rank .. rank + rot) -- the plain
+//     channels reach q_out[m][head][0 .. rank) through the key up-projection, which is another kernel's work;
 //   unit heads: the latent part normed over its `rank` channels (x / sqrt(mean(x^2) + eps) * weight) and the
 //     rotated key part turned, into the token's cache row [rank + rot].
+__device__ __forceinline__ void turn_part(const elem_t* src, elem_t* dst, const float* cs, int rot, int interleaved, int lane) {
+    const int half = rot >> 1;
+    for (int j = lane; j < half; j += 64) {
+        const int a = interleaved ? 2 * j : j, b = interleaved ? 2 * j + 1 : j + half;
+        const float u = to_float(src[a]), v = to_float(src[b]);
+        dst[a] = from_float<elem_t>(turn_x(u, v, cs[j], cs[half + j]));
+        dst[b] = from_float<elem_t>(turn_y(u, v, cs[j], cs[half + j]));
+    }
+}
+
 __global__ __launch_bounds__(64) void latent_prep_kernel(
-    const elem_t* __restrict__ proj, long ld, elem_t* __restrict__ q_out, elem_t* __restrict__ pages, long row_width,
-    const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ slots,
-    const int32_t* __restrict__ positions, const float* __restrict__ norm_w, float eps, const float* __restrict__ rope,
-    int heads, int dim, int rot, int rank, int page_size, int write_cache) {
+    const elem_t* __restrict__ q_src, long q_ld, const elem_t* __restrict__ kv_src, long kv_ld, elem_t* __restrict__ q_out,
+    elem_t* __restrict__ pages, long row_width, const int32_t* __restrict__ block_table, int max_blocks,
+    const int32_t* __restrict__ slots, const int32_t* __restrict__ positions, const float* __restrict__ norm_w, float eps,
+    const float* __restrict__ rope, int heads, int dim, int rot, int rank, int page_size, int write_cache, int interleaved) {
     const int m = blockIdx.x, unit = blockIdx.y, lane = threadIdx.x;
     const int pos = positions[m];
-    const int half = rot >> 1;
     const float* cs = rope + (size_t)pos * rot;
     if (unit < heads) {
-        const elem_t* src = proj + (size_t)m * ld + (size_t)unit * (dim + rot) + dim;
-        elem_t* dst = q_out + ((size_t)m * heads + unit) * (rank + rot) + rank;
-        for (int j = lane; j < half; j += 64) {
-            const float u = to_float(src[j]), v = to_float(src[j + half]);
-            dst[j] = from_float<elem_t>(turn_x(u, v, cs[j], cs[half + j]));
-            dst[j + half] = from_float<elem_t>(turn_y(u, v, cs[j], cs[half + j]));
-        }
+        turn_part(q_src + (size_t)m * q_ld + (size_t)unit * (dim + rot) + dim,
+                  q_out + ((size_t)m * heads + unit) * (rank + rot) + rank, cs, rot, interleaved, lane);
         return;
     }
     if (!write_cache) return;
@@ -227,7 +251,7 @@ __global__ __launch_bounds__(64) void latent_prep_kernel(
     const int page = block < max_blocks ? block_table[(size_t)slots[m] * max_blocks + block] : -1;
     if (page < 0) return;
     elem_t* dst = pages + ((long long)page * page_size + pos % page_size) * row_width;
-    const elem_t* src = proj + (size_t)m * ld + (size_t)heads * (dim + rot);
+    const elem_t* src = kv_src + (size_t)m * kv_ld;
     float sum = 0.f;
     for (int d = lane; d < rank; d += 64) {
         const float x = to_float(src[d]);
@@ -236,11 +260,7 @@ __global__ __launch_bounds__(64) void latent_prep_kernel(
     sum = wave_sum(sum);
     const float r = 1.0f / sqrtf(sum / (float)rank + eps);
     for (int d = lane; d < rank; d += 64) dst[d] = from_float<elem_t>((to_float(src[d]) * r) * norm_w[d]);
-    for (int j = lane; j < half; j += 64) {
-        const float u = to_float(src[rank + j]), v = to_float(src[rank + j + half]);
-        dst[rank + j] = from_float<elem_t>(turn_x(u, v, cs[j], cs[half + j]));
-        dst[rank + j + half] = from_float<elem_t>(turn_y(u, v, cs[j], cs[half + j]));
-    }
+    turn_part(src + rank, dst + rank, cs, rot, interleaved, lane);
 }
 
 #if MLR_BF16
@@ -571,25 +591,27 @@ int mlr_sink_qkv_prep(const void* proj, long ld, const float* bias, void* q_out,
                       void* v_pages, long v_row, const int32_t* block_table, int max_blocks, const int32_t* slots,
                       const int32_t* positions, const float* q_norm_w, const float* k_norm_w, float eps,
                       const float* rope, int rot_dim, int rows, int q_heads, int kv_heads, int key_dim, int value_dim,
-                      int page_size, int write_cache, hipStream_t stream) {
+                      int page_size, int write_cache, int norm_mode, int interleaved, hipStream_t stream) {
     if (rows <= 0) return 0;
-    if (key_dim > MAX_KEY_DIM || q_heads + 2 * kv_heads > 65535 || rot_dim > key_dim || (rot_dim & 1)) return -1;
+    if (key_dim > MAX_KEY_DIM || q_heads + 2 * kv_heads > 65535 || rot_dim > key_dim || (rot_dim & 1) || norm_mode < 0 ||
+        norm_mode > 2)
+        return -1;
     sink_qkv_prep_kernel<<<dim3(rows, q_heads + 2 * kv_heads), 64, 0, stream>>>(
         (const elem_t*)proj, ld, bias, (elem_t*)q_out, (elem_t*)k_pages, k_row, (elem_t*)v_pages, v_row, block_table,
         max_blocks, slots, positions, q_norm_w, k_norm_w, eps, rope, rot_dim, q_heads, kv_heads, key_dim, value_dim,
-        page_size, write_cache);
+        page_size, write_cache, norm_mode, interleaved);
     return (int)hipGetLastError();
 }
 
-int mlr_latent_prep(const void* proj, long ld, void* q_out, void* pages, long row_width, const int32_t* block_table,
-                    int max_blocks, const int32_t* slots, const int32_t* positions, const float* norm_w, float eps,
-                    const float* rope, int rows, int heads, int dim, int rot, int rank, int page_size, int write_cache,
-                    hipStream_t stream) {
+int mlr_latent_prep(const void* q_src, long q_ld, const void* kv_src, long kv_ld, void* q_out, void* pages, long row_width,
+                    const int32_t* block_table, int max_blocks, const int32_t* slots, const int32_t* positions,
+                    const float* norm_w, float eps, const float* rope, int rows, int heads, int dim, int rot, int rank,
+                    int page_size, int write_cache, int interleaved, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (heads + 1 > 65535 || (rot & 1) || rot <= 0 || rope == nullptr) return -1;
     latent_prep_kernel<<<dim3(rows, heads + 1), 64, 0, stream>>>(
-        (const elem_t*)proj, ld, (elem_t*)q_out, (elem_t*)pages, row_width, block_table, max_blocks, slots, positions,
-        norm_w, eps, rope, heads, dim, rot, rank, page_size, write_cache);
+        (const elem_t*)q_src, q_ld, (const elem_t*)kv_src, kv_ld, (elem_t*)q_out, (elem_t*)pages, row_width, block_table,
+        max_blocks, slots, positions, norm_w, eps, rope, heads, dim, rot, rank, page_size, write_cache, interleaved);
     return (int)hipGetLastError();
 }
 

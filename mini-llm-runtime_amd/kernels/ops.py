@@ -224,6 +224,73 @@ class Kernels:
         fn = self._lib("elementwise").mlr_silu_mul
         _ok(fn(_p(gate_up), _p(act), _c_int(m), _c_int(two_f // 2), _stream()), "silu_mul")
 
+    GATED_ACTS = {"silu": 0, "gelu_tanh": 1}
+
+    @timed("activation", _tensors_work())
+    def gated_act_mul(self, gate_up, act, kind):
+        """act[m, f] = kind(gate_up[m, f]) * gate_up[m, F + f]; kind: silu, or gelu_tanh,
+        0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3)))."""
+        _need(kind in self.GATED_ACTS, f"gated_act_mul: activation {kind!r} ({', '.join(self.GATED_ACTS)})")
+        _tensor(gate_up, "gate_up", self.dtype, ndim=2)
+        m, two_f = gate_up.shape
+        _need(two_f % 2 == 0, "gate_up: the width must be even")
+        _tensor(act, "act", self.dtype, (m, two_f // 2))
+        _ok(self._lib("elementwise").mlr_gated_act_mul(_p(gate_up), _p(act), _c_int(m), _c_int(two_f // 2),
+                                                       _c_int(self.GATED_ACTS[kind]), _stream()), "gated_act_mul")
+
+    @timed("embed", _tensors_work())
+    def pair_embed(self, ids, positions, slots, table, pairs, live, stage, h, buckets, mul_prev, mul_cur):
+        """h[m] = float(table[ids[m]]) + float(pairs[row]), row = (token before * mul_prev + ids[m] * mul_cur) mod
+        buckets, or row `buckets` at position 0.  The token before: the row above when it is the same request's
+        previous position, else live[slot] (int32 [slots, 1]); a request's last row leaves its token in stage[slot]."""
+        rows = ids.numel()
+        for name, t in (("ids", ids), ("positions", positions), ("slots", slots)):
+            _tensor(t, name, torch.int32, (rows,))
+        _tensor(table, "table", self.dtype, ndim=2)
+        vocab, width = table.shape
+        _tensor(pairs, "pairs", self.dtype, (buckets + 1, width))
+        _tensor(live, "live", torch.int32, ndim=2)
+        _tensor(stage, "stage", torch.int32, tuple(live.shape))
+        _need(live.shape[1] == 1 and buckets >= 1, "pair_embed: one token a slot, and at least one bucket")
+        _tensor(h, "h", torch.float32, (rows, width))
+        _ok(self._lib("elementwise").mlr_pair_embed(_p(ids), _p(positions), _p(slots), _p(table), _p(pairs), _p(live),
+                                                    _p(stage), _p(h), _c_int(rows), _c_int(width), _c_int(vocab),
+                                                    _c_int(buckets), ctypes.c_longlong(mul_prev), ctypes.c_longlong(mul_cur),
+                                                    _stream()), "pair_embed")
+
+    GATE_KINDS = {"silu": 0, "sigmoid": 1}
+
+    @timed("activation", _tensors_work())
+    def gate_mul(self, x, gate, out, kind="sigmoid", scale=1.0):
+        """out = scale * x * kind(gate); gate: columns of a row-major matrix; out may be x."""
+        _tensor(x, "x", self.dtype, ndim=2)
+        m, width = x.shape
+        stride = self._columns(gate, "gate", self.dtype, m, width)
+        _tensor(out, "out", self.dtype, (m, width))
+        _need(kind in self.GATE_KINDS, f"gate_mul: gate {kind!r}")
+        _ok(self._lib("elementwise").mlr_gate_mul(_p(x), _p(gate), ctypes.c_long(stride), _p(out), _c_int(m), _c_int(width),
+                                                  _c_int(self.GATE_KINDS[kind]), _c_float(scale), _stream()), "gate_mul")
+
+    @timed("norm", _tensors_work())
+    def rmsnorm_columns(self, x, weight, out, eps):
+        """out = x / sqrt(mean(x^2) + eps) * weight, row by row, x being columns of a row-major matrix; 32-bit inside."""
+        _need(isinstance(x, torch.Tensor) and x.dim() == 2, "rmsnorm_columns: x must be a matrix")
+        rows, width = x.shape
+        stride = self._columns(x, "x", self.dtype, rows, width)
+        _tensor(weight, "weight", torch.float32, (width,))
+        _tensor(out, "out", self.dtype, (rows, width))
+        _ok(self._lib("elementwise").mlr_rmsnorm_columns(_p(x), ctypes.c_long(stride), _p(weight), _p(out), _c_int(rows),
+                                                         _c_int(width), _c_float(eps), _stream()), "rmsnorm_columns")
+
+    @timed("norm", _tensors_work())
+    def scaled_sum(self, a, b, out, sa, sb):
+        """out = sa * a + sb * b, the sum taken in 32-bit; out may be a or b."""
+        _tensor(a, "a", self.dtype)
+        _tensor(b, "b", self.dtype, tuple(a.shape))
+        _tensor(out, "out", self.dtype, tuple(a.shape))
+        _ok(self._lib("elementwise").mlr_scaled_sum(_p(a), _p(b), _p(out), _c_float(sa), _c_float(sb), _c_size_t(a.numel()),
+                                                    _stream()), "scaled_sum")
+
     # -- projections -------------------------------------------------------------------------
     @timed("gemm", _gemm_work)
     def gemm(self, a, w, out):
@@ -799,7 +866,7 @@ class Kernels:
     @timed("recurrence", _tensors_work())
     def linear_recurrence(self, q, k, v, log_decay, out, live, stage, state_offset, seg_first, seg_count, segments, slots,
                           heads, n_keys, n_values, heads_per_group=1, v_scale=None, skip=None, q_scale=1.0,
-                          write_state=True, piece_state=None, piece_decay=None):
+                          write_state=True, piece_state=None, piece_decay=None, activation=None):
         """Per request of the step and head, from the live state: S_t = diag(exp(log_decay_t)) S_(t-1) + k_t (v_scale_t
         v_t)^T, out_t = S_t^T (q_scale q_t) + skip[head] v_t.  q, k: columns [rows, (heads / heads_per_group) * n_keys];
         v: columns [rows, heads * n_values]; log_decay float [rows, heads * n_keys] (a decay per key channel) or
@@ -807,7 +874,8 @@ class Kernels:
         `state_offset` on in a slot's row of `live`/`stage`.
         With `piece_state` float [segments * heads * n_keys * n_values] and `piece_decay` float [segments * heads *
         n_keys]: `seg_first`/`seg_count` name PIECES of requests (a request's pieces one after the other), which run
-        side by side in three passes; the result differs from the token-by-token order by 32-bit rounding."""
+        side by side in three passes; the result differs from the token-by-token order by 32-bit rounding.
+        log_decay float [heads]: one constant decay a head.  `activation` "silu": q, k and v pass it as they are read."""
         rows = v.shape[0]
         groups = heads // heads_per_group
         _need(heads >= 1 and heads_per_group >= 1 and heads % heads_per_group == 0, "linear_recurrence: heads and groups")
@@ -815,11 +883,18 @@ class Kernels:
         qs = self._columns(q, "q", self.dtype, rows, groups * n_keys)
         ks = self._columns(k, "k", self.dtype, rows, groups * n_keys)
         vs = self._columns(v, "v", self.dtype, rows, heads * n_values)
-        _tensor(log_decay, "log_decay", torch.float32, ndim=2)
-        per_channel = log_decay.shape[1] == heads * n_keys and not (n_keys == 1 and False)
-        _need(tuple(log_decay.shape) in ((rows, heads * n_keys), (rows, heads)), "log_decay: [rows, heads * keys] or [rows, heads]")
-        if n_keys == 1:
-            per_channel = True                  # (the two layouts coincide)
+        _need(activation in (None, "silu"), f"linear_recurrence: activation {activation!r}")
+        if log_decay.dim() == 1:                # the same decays for every token
+            _tensor(log_decay, "log_decay", torch.float32, (heads,))
+            per_channel, decay_stride = False, 0
+        else:
+            _tensor(log_decay, "log_decay", torch.float32, ndim=2)
+            per_channel = log_decay.shape[1] == heads * n_keys
+            _need(tuple(log_decay.shape) in ((rows, heads * n_keys), (rows, heads)),
+                  "log_decay: [rows, heads * keys], [rows, heads] or [heads]")
+            decay_stride = log_decay.shape[1]
+            if n_keys == 1:
+                per_channel = True              # (the two layouts coincide)
         if v_scale is not None:
             _tensor(v_scale, "v_scale", torch.float32, (rows, heads))
         if skip is not None:
@@ -839,12 +914,58 @@ class Kernels:
         fn = self._lib("recurrence").mlr_linear_recurrence
         at = state_offset * 4
         _ok(fn(_p(q), ctypes.c_long(qs), _p(k), ctypes.c_long(ks), _p(v), ctypes.c_long(vs), _p(log_decay),
-               ctypes.c_long(log_decay.shape[1]), _c_int(1 if per_channel else 0), _p(v_scale),
+               ctypes.c_long(decay_stride), _c_int(1 if per_channel else 0), _p(v_scale),
                ctypes.c_long(heads if v_scale is not None else 0), _p(skip), _c_float(q_scale), _p(out),
                _ptr(live.data_ptr() + at), _ptr(stage.data_ptr() + at), ctypes.c_long(live.stride(0)), _p(seg_first),
                _p(seg_count), _p(slots), _c_int(segments), _c_int(heads), _c_int(heads_per_group), _c_int(n_keys),
-               _c_int(n_values), _c_int(1 if write_state else 0), _p(piece_state), _p(piece_decay), _stream()),
-            "linear_recurrence")
+               _c_int(n_values), _c_int(1 if write_state else 0), _p(piece_state), _p(piece_decay),
+               _c_int(1 if activation == "silu" else 0), _stream()), "linear_recurrence")
+
+    @timed("activation", _tensors_work())
+    def channel_log_decay(self, z, bias, a_log, out, heads, n_keys):
+        """out = -exp(a_log[head]) * softplus(z + bias): the logarithm of a decay per key channel, 32-bit;
+        z float [rows, heads * n_keys], bias float [heads * n_keys] or None, a_log float [heads]."""
+        _tensor(z, "z", torch.float32, ndim=2)
+        rows = z.shape[0]
+        _need(z.shape[1] == heads * n_keys, "channel_log_decay: z must be [rows, heads * keys]")
+        if bias is not None:
+            _tensor(bias, "bias", torch.float32, (heads * n_keys,))
+        _tensor(a_log, "a_log", torch.float32, (heads,))
+        _tensor(out, "out", torch.float32, (rows, heads * n_keys))
+        _ok(self._lib("recurrence").mlr_channel_log_decay(_p(z), _p(bias), _p(a_log), _p(out), _c_int(rows), _c_int(heads),
+                                                          _c_int(n_keys), _stream()), "channel_log_decay")
+
+    @timed("recurrence", _tensors_work())
+    def delta_rule(self, q, k, v, log_decay, beta_raw, out, live, stage, state_offset, seg_first, seg_count, segments, slots,
+                   heads, n_keys, n_values, heads_per_group=1, q_scale=1.0, unit_norm=True, unit_eps=1e-6, write_state=True):
+        """Per request of the step and head, from the live state: S <- diag(exp(log_decay_t)) S; u = beta_t (v_t - S^T k_t);
+        S <- S + k_t u^T; out_t = S^T q_t, with beta = sigmoid(beta_raw).  q, k: columns [rows, (heads / heads_per_group) *
+        n_keys], made unit vectors per head inside (x / sqrt(sum x^2 + unit_eps); `unit_norm` False: taken as they
+        are) and q multiplied by q_scale; v: columns [rows, heads * n_values]; log_decay float [rows, heads * n_keys];
+        beta_raw float columns [rows, heads]; the state [heads][n_keys][n_values] floats from `state_offset` on in a
+        slot's row of `live`/`stage`."""
+        rows = v.shape[0]
+        _need(heads >= 1 and heads_per_group >= 1 and heads % heads_per_group == 0, "delta_rule: heads and groups")
+        groups = heads // heads_per_group
+        _need(1 <= n_keys <= self.RECURRENCE_MAX_KEYS, f"delta_rule: 1..{self.RECURRENCE_MAX_KEYS} key channels a head")
+        qs = self._columns(q, "q", self.dtype, rows, groups * n_keys)
+        ks = self._columns(k, "k", self.dtype, rows, groups * n_keys)
+        vs = self._columns(v, "v", self.dtype, rows, heads * n_values)
+        _tensor(log_decay, "log_decay", torch.float32, (rows, heads * n_keys))
+        bs = self._columns(beta_raw, "beta_raw", torch.float32, rows, heads)
+        _tensor(out, "out", torch.float32, (rows, heads * n_values))
+        self._check_state(live, stage, state_offset, heads * n_keys * n_values)
+        _tensor(seg_first, "seg_first", torch.int32, (segments,))
+        _tensor(seg_count, "seg_count", torch.int32, (segments,))
+        _tensor(slots, "slots", torch.int32, (rows,))
+        _need(segments <= 65535 * 32 and heads <= 65535, "delta_rule: too many requests or heads for the grid")
+        at = state_offset * 4
+        _ok(self._lib("recurrence").mlr_delta_rule(
+            _p(q), ctypes.c_long(qs), _p(k), ctypes.c_long(ks), _p(v), ctypes.c_long(vs), _p(log_decay), _p(beta_raw),
+            ctypes.c_long(bs), _p(out), _ptr(live.data_ptr() + at), _ptr(stage.data_ptr() + at), ctypes.c_long(live.stride(0)),
+            _p(seg_first), _p(seg_count), _p(slots), _c_int(segments), _c_int(heads), _c_int(heads_per_group), _c_int(n_keys),
+            _c_int(n_values), _c_int(1 if write_state else 0), _c_int(1 if unit_norm else 0), _c_float(q_scale),
+            _c_float(unit_eps), _stream()), "delta_rule")
 
     # -- differential attention -----------------------------------------------------------------------
     DIFF_MAX_HEAD_DIM = 256
@@ -1043,15 +1164,17 @@ class Kernels:
 
     @timed("rope_kv", _rope_work)
     def sink_qkv_prep(self, proj, bias, q_out, k_pages, v_pages, block_table, slots, positions, q_norm_w, k_norm_w, eps,
-                      rope, q_heads, kv_heads, key_dim, value_dim, page_size, write_cache=True):
-        """From the stacked projection [rows, q_heads * key_dim + kv_heads * (key_dim + value_dim)]: bias (float, may be
-        None), per-head RMSNorm of q and k (weights may be None), rotation of a head's first rope.shape[1] channels
-        in pairs (j, j + half) (rope float [positions, rot]: cosines | sines; may be None); q to q_out, k and v into
-        their row-major pages."""
+                      rope, q_heads, kv_heads, key_dim, value_dim, page_size, write_cache=True, norm="auto",
+                      interleaved=False):
+        """From the stacked projection [rows, q_heads * key_dim + kv_heads * (key_dim + value_dim)] (further columns behind these are left alone): bias (float, may be
+        None), per-head RMSNorm of q and k, rotation of a head's first rope.shape[1] channels in pairs (j, j + half)
+        or, `interleaved`, (2 j, 2 j + 1) (rope float [positions, rot]: cosines | sines; may be None); q to q_out, k
+        and v into their row-major pages.  `norm`: "before" the rotation, "after" it, None, or "auto" (before it when
+        weights are given, else none); the weights may be None with any of them (a norm without a weight)."""
         total = q_heads * key_dim + kv_heads * (key_dim + value_dim)
         _tensor(proj, "proj", self.dtype, ndim=2)
         rows = proj.shape[0]
-        _need(proj.shape[1] == total, lambda: f"proj: expected width {total}, got {proj.shape[1]}")
+        _need(proj.shape[1] >= total, lambda: f"proj: expected a width of at least {total}, got {proj.shape[1]}")
         if bias is not None:
             _tensor(bias, "bias", torch.float32, (total,))
         _tensor(q_out, "q_out", self.dtype, (rows, q_heads * key_dim))
@@ -1069,22 +1192,35 @@ class Kernels:
             _tensor(rope, "rope", torch.float32, ndim=2)
             rot = rope.shape[1]
             _need(2 <= rot <= key_dim and rot % 2 == 0, f"rope: the table's width {rot} must be even and at most {key_dim}")
+        if norm == "auto":
+            norm = "before" if q_norm_w is not None else None
+        _need(norm in (None, "before", "after"), f"sink_qkv_prep: norm {norm!r}")
+        mode = {None: 0, "before": 1, "after": 2}[norm]
         _ok(self._lib("sink_attention").mlr_sink_qkv_prep(
-            _p(proj), ctypes.c_long(total), _p(bias), _p(q_out), _p(k_pages), ctypes.c_long(k_row), _p(v_pages),
+            _p(proj), ctypes.c_long(proj.shape[1]), _p(bias), _p(q_out), _p(k_pages), ctypes.c_long(k_row), _p(v_pages),
             ctypes.c_long(v_row), _p(block_table), _c_int(block_table.shape[1]), _p(slots), _p(positions), _p(q_norm_w),
             _p(k_norm_w), _c_float(eps), _p(rope), _c_int(rot), _c_int(rows), _c_int(q_heads), _c_int(kv_heads),
-            _c_int(key_dim), _c_int(value_dim), _c_int(page_size), _c_int(1 if write_cache else 0), _stream()),
-            "sink_qkv_prep")
+            _c_int(key_dim), _c_int(value_dim), _c_int(page_size), _c_int(1 if write_cache else 0), _c_int(mode),
+            _c_int(1 if interleaved else 0), _stream()), "sink_qkv_prep")
 
     @timed("rope_kv", _rope_work)
     def latent_prep(self, proj, q_out, pages, block_table, slots, positions, norm_w, eps, rope, heads, dim, rot, rank,
-                    page_size, write_cache=True):
+                    page_size, write_cache=True, q_src=None, interleaved=False):
         """Latent attention's row work on proj [rows, heads * (dim + rot) + rank + rot]: every head's rotated query
         channels turned into q_out[:, head, rank:], the latent part normed and the shared rotated key part turned
-        into the token's cache row [rank + rot] of pages [pages, 1, page, rank + rot]."""
-        _tensor(proj, "proj", self.dtype, ndim=2)
+        into the token's cache row [rank + rot] of pages [pages, 1, page, rank + rot].  With `q_src` (columns
+        [rows, heads * (dim + rot)]) the queries come from there and proj holds [rows, rank + rot] only.  The rotated
+        parts turn in pairs (j, j + rot / 2) or, `interleaved`, (2 j, 2 j + 1)."""
         rows = proj.shape[0]
-        _need(proj.shape[1] == heads * (dim + rot) + rank + rot, "proj: wrong width")
+        if q_src is None:
+            _tensor(proj, "proj", self.dtype, ndim=2)
+            _need(proj.shape[1] == heads * (dim + rot) + rank + rot, "proj: wrong width")
+            q_ptr, q_ld = proj.data_ptr(), proj.shape[1]
+            kv_ptr, kv_ld = proj.data_ptr() + heads * (dim + rot) * proj.element_size(), proj.shape[1]
+        else:
+            q_ld = self._columns(q_src, "q_src", self.dtype, rows, heads * (dim + rot))
+            kv_ld = self._columns(proj, "proj", self.dtype, rows, rank + rot)
+            q_ptr, kv_ptr = q_src.data_ptr(), proj.data_ptr()
         _tensor(q_out, "q_out", self.dtype, (rows, heads * (rank + rot)))
         _need(self._sink_pages(pages, "pages", 1, page_size, rank + rot) == rank + rot, "pages: rows of rank + rot")
         _tensor(block_table, "block_table", torch.int32, ndim=2)
@@ -1094,10 +1230,10 @@ class Kernels:
         _tensor(rope, "rope", torch.float32, ndim=2)
         _need(rope.shape[1] == rot and rot % 2 == 0 and rot >= 2, "rope: as wide as the rotated part, which is even")
         _ok(self._lib("sink_attention").mlr_latent_prep(
-            _p(proj), ctypes.c_long(proj.shape[1]), _p(q_out), _p(pages), ctypes.c_long(rank + rot), _p(block_table),
-            _c_int(block_table.shape[1]), _p(slots), _p(positions), _p(norm_w), _c_float(eps), _p(rope), _c_int(rows),
-            _c_int(heads), _c_int(dim), _c_int(rot), _c_int(rank), _c_int(page_size), _c_int(1 if write_cache else 0),
-            _stream()), "latent_prep")
+            _ptr(q_ptr), ctypes.c_long(q_ld), _ptr(kv_ptr), ctypes.c_long(kv_ld), _p(q_out), _p(pages),
+            ctypes.c_long(rank + rot), _p(block_table), _c_int(block_table.shape[1]), _p(slots), _p(positions), _p(norm_w),
+            _c_float(eps), _p(rope), _c_int(rows), _c_int(heads), _c_int(dim), _c_int(rot), _c_int(rank), _c_int(page_size),
+            _c_int(1 if write_cache else 0), _c_int(1 if interleaved else 0), _stream()), "latent_prep")
 
     @timed("attention")
     def sink_attention(self, q, k_pages, v_pages, block_table, slots, positions, sink, out, q_heads, kv_heads, key_dim,

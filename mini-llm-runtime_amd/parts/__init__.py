@@ -1,4 +1,4 @@
-from . import attention, block, diff_attention, ends, mlp, norm, recurrent, rope, routed, sink_attention  # noqa: F401  (they register themselves)
+from . import attention, block, combine, diff_attention, ends, mlp, norm, recurrent, rope, routed, sink_attention  # noqa: F401  (they register themselves)
 from .model import DecoderModel, build_blocks, expected_tensors
 from .registry import PartError, build_part, part_class, register_part
 

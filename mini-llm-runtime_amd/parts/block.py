@@ -1,7 +1,7 @@
 """Arrangement of the parts in a layer.  Pre-norm residual block (src/minillm/runtime.cpp:245-337):
 h += mixer(norm1(h)); h += ffn(norm2(h)).  The residual stream h is float; every add into it is
 fused with the norm that follows, so a block hands its last output on as `pending` instead of
-adding it itself."""
+adding it itself.  `norm2` and `ffn` may be missing: a layer of the first sublayer only."""
 from __future__ import annotations
 
 from .registry import Complete, Handoff, build_part, register_part
@@ -13,11 +13,16 @@ class PreNormBlock:
     def __init__(self, spec):
         self.norm1 = build_part("norm", spec.norm1)
         self.mixer = build_part("mixer", spec.mixer)
-        self.norm2 = build_part("norm", spec.norm2)
-        self.ffn = build_part("ffn", spec.ffn)
+        if (spec.ffn is None) != (spec.norm2 is None):
+            raise ValueError("a pre-norm block has a feed-forward and its norm, or neither")
+        self.norm2 = build_part("norm", spec.norm2) if spec.norm2 is not None else None
+        self.ffn = build_part("ffn", spec.ffn) if spec.ffn is not None else None
 
     def parts(self):
-        return {"norm1": self.norm1, "mixer": self.mixer, "norm2": self.norm2, "ffn": self.ffn}
+        out = {"norm1": self.norm1, "mixer": self.mixer}
+        if self.ffn is not None:
+            out.update(norm2=self.norm2, ffn=self.ffn)
+        return out
 
     def workspace_plan(self, rows, dtype, limits):
         import torch
@@ -29,7 +34,8 @@ class PreNormBlock:
     def forward(self, ctx, h, pending, cache_id, write_cache=True, next_norm=None):
         fusable = lambda norm: norm is not None and getattr(norm, "fusable_rmsnorm", False) and norm.size == h.shape[1]
         if (ctx.kernels.handoff_supported(h.shape[0]) and fusable(self.norm1) and fusable(self.norm2)
-                and hasattr(self.mixer, "forward_handoff") and hasattr(self.ffn, "forward_handoff")):
+                and getattr(self.mixer, "forward_handoff", None) is not None
+                and getattr(self.ffn, "forward_handoff", None) is not None):
             # few rows: every norm is shared between the projection before it (which adds into h and leaves
             # h * weight and partial sums of squares) and the projection after it (which applies the scale)
             hand = pending if isinstance(pending, Handoff) and pending.norm is self.norm1 else \
@@ -41,6 +47,8 @@ class PreNormBlock:
         normed = ctx.workspace.get("normed", tuple(h.shape), ctx.dtype)
         self.norm1.forward(ctx, h, pending, normed)
         mixed = self.mixer.forward(ctx, normed, cache_id, write_cache)
+        if self.ffn is None:
+            return mixed                                  # (whoever norms next adds it)
         self.norm2.forward(ctx, h, mixed, normed)
         return self.ffn.forward(ctx, normed)
 

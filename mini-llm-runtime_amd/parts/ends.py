@@ -8,11 +8,12 @@ from __future__ import annotations
 
 import torch
 
+from ..cache.manager import StateSpec
 from ..config.specs import EmbedSpec, HeadSpec
 from ..weights.loader import WeightSpec
 from .registry import PartError, register_part
 
-__all__ = ["TokenEmbedding", "LinearHead", "ScaledHead", "EmbedSpec", "HeadSpec"]
+__all__ = ["TokenEmbedding", "PairEmbedding", "LinearHead", "ScaledHead", "EmbedSpec", "HeadSpec"]
 
 
 @register_part("embed", "token_embedding")
@@ -45,6 +46,41 @@ class TokenEmbedding:
         """The float residual stream [B, E] of the step's tokens."""
         h = ctx.workspace.get("hidden", (ctx.n_tokens, self.spec.hidden), torch.float32)
         ctx.kernels.embed_gather(ctx.token_ids, self.weight, h)
+        return h
+
+
+@register_part("embed", "pair_embedding")
+class PairEmbedding(TokenEmbedding):
+    """A token's embedding plus a row of a second table that the token and the one before it pick:
+    row (previous * mul_prev + token * mul_cur) mod buckets, and the table's last row (number `buckets`) for a
+    request's first token.  The token before a step's first token of a request is state of the request: an embedding
+    with a `cache_spec()` gets a cache entry like a mixer does (`cache_id`, set by the model), here one integer a
+    slot, staged by the last row a request brings and made live with every other state when the step has run."""
+    graph_safe = True
+
+    def __init__(self, spec):
+        super().__init__(spec)
+        if spec.buckets < 1:
+            raise PartError("the pair table needs at least one bucket")
+        self.pairs = None
+        self.cache_id = None
+
+    def weight_specs(self):
+        s = self.spec
+        return {"weight": WeightSpec((s.vocab_size, s.hidden)), "pairs": WeightSpec((s.buckets + 1, s.hidden))}
+
+    def bind(self, weights):
+        self.weight, self.pairs = weights["weight"], weights["pairs"]
+
+    def cache_spec(self):
+        return StateSpec((1,), torch.int32)
+
+    def forward(self, ctx):
+        s = self.spec
+        h = ctx.workspace.get("hidden", (ctx.n_tokens, s.hidden), torch.float32)
+        ctx.kernels.pair_embed(ctx.token_ids, ctx.positions, ctx.slots, self.weight, self.pairs,
+                               ctx.cache.state_view(self.cache_id), ctx.cache.state_stage(self.cache_id), h,
+                               s.buckets, s.mul_prev, s.mul_cur)
         return h
 
 

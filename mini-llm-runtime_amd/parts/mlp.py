@@ -1,5 +1,6 @@
 """SwiGLU feed-forward: out = (silu(x Wgate^T) * (x Wup^T)) Wdown^T with silu(g) = g / (1 + exp(-g))
-(src/minillm/runtime.cpp:323-336).  Gate and up are one stacked projection."""
+(src/minillm/runtime.cpp:323-336).  Gate and up are one stacked projection.  The gate's activation is the spec's:
+silu, or gelu_tanh (0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))), which takes the unfused path."""
 from __future__ import annotations
 
 import torch
@@ -12,11 +13,13 @@ from .registry import Handoff, PartError, register_part
 class SwiGluMlp:
     graph_safe = True        # forward launches kernels over the step's device vectors only
     def __init__(self, spec):
-        if spec.activation != "silu":
-            raise PartError(f"activation {spec.activation!r} is not built (silu)")
+        if spec.activation not in ("silu", "gelu_tanh"):
+            raise PartError(f"activation {spec.activation!r} is not built (silu, gelu_tanh)")
         self.spec = spec
         self.gate_up = None
         self.down = None
+        if spec.activation != "silu":         # the projections' fused epilogues are silu's
+            self.forward_handoff = None
 
     def weight_specs(self):
         s = self.spec
@@ -56,12 +59,15 @@ class SwiGluMlp:
         s = self.spec
         m = x.shape[0]
         act = ctx.workspace.get("act", (m, s.intermediate), x.dtype)
-        if ctx.kernels.gated_silu_fused(m, s.hidden):  # few rows: the activation rides on the projection
-            ctx.kernels.gemm_gated_silu(x, self.gate_up, act)
+        if s.activation == "silu" and ctx.kernels.gated_silu_fused(m, s.hidden):
+            ctx.kernels.gemm_gated_silu(x, self.gate_up, act)      # few rows: the activation rides on the projection
         else:
             gate_up = ctx.workspace.get("gate_up", (m, 2 * s.intermediate), x.dtype)
             ctx.kernels.gemm(x, self.gate_up, gate_up)
-            ctx.kernels.silu_mul(gate_up, act)
+            if s.activation == "silu":
+                ctx.kernels.silu_mul(gate_up, act)
+            else:
+                ctx.kernels.gated_act_mul(gate_up, act, s.activation)
         out = ctx.workspace.get("ffn_out", (m, s.hidden), x.dtype)
         ctx.kernels.gemm(act, self.down, out)
         return out

@@ -73,21 +73,37 @@ class DecoderModel:
         for i, block in enumerate(self.blocks):
             for part_name, part in block.parts().items():
                 part.bind(by_owner.get((i, part_name), {}))
-        # cache entries: one per cache id the schedule names
+        # cache entries: one per cache id the schedule names.  A mixer that is several mixers side by side names
+        # a tuple of needs: its first entry takes the run's cache id, the others get ids beyond the schedule's, and
+        # its forward is handed the tuple of ids.  An embedding with state of its own gets one more entry.
         n_entries = 1 + max(run.cache for run in spec.schedule)
         self.cache_entry_specs = [None] * n_entries
+        self.cache_ids = {}                   # the schedule's cache id -> what the block is handed (an id or a tuple)
+        needs = {}
         writers = set()
         for run in spec.schedule:
             cs = self.blocks[run.layer].mixer.cache_spec()
-            if self.cache_entry_specs[run.cache] is None:
-                self.cache_entry_specs[run.cache] = cs
-            elif self.cache_entry_specs[run.cache] != cs:
+            if run.cache not in needs:
+                needs[run.cache] = cs
+                if isinstance(cs, tuple):
+                    ids = [run.cache] + list(range(len(self.cache_entry_specs), len(self.cache_entry_specs) + len(cs) - 1))
+                    self.cache_entry_specs += [None] * (len(cs) - 1)
+                    for cid, sub in zip(ids, cs):
+                        self.cache_entry_specs[cid] = sub
+                    self.cache_ids[run.cache] = tuple(ids)
+                else:
+                    self.cache_entry_specs[run.cache] = cs
+                    self.cache_ids[run.cache] = run.cache
+            elif needs[run.cache] != cs:
                 raise PartError(f"cache entry {run.cache} is shared by mixers with different needs")
             if run.write_cache:
                 writers.add(run.cache)
         for cid in range(n_entries):
-            if self.cache_entry_specs[cid] is not None and cid not in writers:
+            if needs.get(cid) not in (None, ()) and cid not in writers:
                 raise PartError(f"cache entry {cid} is read but never written")
+        if hasattr(self.embed, "cache_spec"):
+            self.embed.cache_id = len(self.cache_entry_specs)
+            self.cache_entry_specs.append(self.embed.cache_spec())
 
     @classmethod
     def load(cls, folder, dtype, device="cuda:0", device_budget_bytes=None):
@@ -166,7 +182,7 @@ class DecoderModel:
             next_norm = next_block.norm1 if next_block is not None else None
             block = self.blocks[run.layer]
             more = {"next_block": next_block} if getattr(block, "wants_next_block", False) else {}
-            pending = block.forward(ctx, h, pending, run.cache, run.write_cache, next_norm=next_norm, **more)
+            pending = block.forward(ctx, h, pending, self.cache_ids[run.cache], run.write_cache, next_norm=next_norm, **more)
             if isinstance(pending, Complete) and i + 1 == len(schedule):
                 pending = None                            # (h is complete)
             if status is not None:                        # h + pending is the hidden state after this run

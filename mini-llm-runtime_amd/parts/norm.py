@@ -1,6 +1,7 @@
 """RMSNorm: y = (x * rsqrt(mean(x^2) + eps)) * w, the weight multiplying directly
 (src/minillm/kernels.cpp:209-216).  The residual add that precedes a norm in the layer is
-fused into the same kernel."""
+fused into the same kernel.  A spec with a `weight_offset` stores its weight as the factor's distance from
+that offset (a weight "around zero": factor 1 + w); the factor is formed once, in 32-bit, when the weights are bound."""
 from __future__ import annotations
 
 import torch
@@ -15,13 +16,15 @@ class RmsNorm:
     fusable_rmsnorm = True   # the projections before and after it may share this norm between them (weight, eps as here)
     def __init__(self, spec):
         self.size, self.eps = spec.size, float(spec.eps)
+        self.offset = float(getattr(spec, "weight_offset", 0.0))
         self.weight = None
 
     def weight_specs(self):
-        return {"weight": WeightSpec((self.size,), keep_float32=True)}
+        init = ("normal", 0.0, 0.1) if self.offset != 0.0 else None
+        return {"weight": WeightSpec((self.size,), keep_float32=True, init=init)}
 
     def bind(self, weights):
-        self.weight = weights["weight"]
+        self.weight = weights["weight"] if self.offset == 0.0 else (weights["weight"].float() + self.offset).contiguous()
 
     def libraries(self):
         return ["elementwise"]

@@ -1,8 +1,10 @@
-"""Mixers that keep a state of fixed size per request instead of keys and values: gated linear attention and
-Mamba-2.  Both run the same recurrence per head,
+"""Mixers that keep a state of fixed size per request instead of keys and values: gated linear attention,
+Mamba-2, linear attention with a constant decay a head, and the gated delta rule.  The first three run the same
+recurrence per head,
     S_t = diag(a_t) S_(t-1) + k_t v_t^T,    o_t = S_t^T q_t       (S: key channels x value channels, 32-bit),
 token by token from the state that earlier steps left (`Kernels.linear_recurrence`); they differ in where q, k,
-v and the decay a come from and in what happens to o.  The state of a request lives in the cache manager's
+v and the decay a come from and in what happens to o.  The delta rule's write first takes back what the state
+holds for the token's key (`Kernels.delta_rule`).  The state of a request lives in the cache manager's
 slots (`StateSpec`): read from the live rows, written to the staged ones, which become live when every layer of
 the step has run."""
 from __future__ import annotations
@@ -206,4 +208,178 @@ class Mamba2:
         k.gated_part_norm(y, z, self.norm, normed, inner // s.norm_groups, float(s.eps), gate_first=True, gate_kind="silu")
         out = ws.get("mixer_out", (m, s.hidden), x.dtype)
         k.gemm(normed, self.o, out)
+        return out
+
+
+@register_part("mixer", "decayed_linear_attention")
+class DecayedLinearAttention:
+    """q = act(Wq x), k = act(Wk x) (heads x head_dim), v = act(Wv x) (heads x value_dim); per head the recurrence
+    above with ONE constant decay a head on every key channel, no other factor; the heads side by side are RMS-normed
+    as one row with a weight as wide as the row, multiplied by gate(Wg x) and projected by Wo."""
+    graph_safe = True
+
+    def __init__(self, spec):
+        s = self.spec = spec
+        if not 1 <= s.head_dim <= 256:
+            raise PartError(f"head_dim {s.head_dim}: the recurrence kernel takes up to 256 key channels a head")
+        if len(s.decay) != s.heads or not all(0.0 < float(d) <= 1.0 for d in s.decay):
+            raise PartError(f"decay: one number in (0, 1] for each of the {s.heads} heads")
+        if s.activation not in (None, "silu") or s.gate not in ("sigmoid", "silu"):
+            raise PartError(f"activation {s.activation!r} / gate {s.gate!r}: silu or none / sigmoid or silu")
+        self.qk_width, self.v_width = s.heads * s.head_dim, s.heads * s.value_dim
+        self.out_name = "mixer_out"
+        self.proj = self.norm = self.o = self._log_decay = None
+
+    def weight_specs(self):
+        s = self.spec
+        return {"q": WeightSpec((self.qk_width, s.hidden), stack="qkvg"), "k": WeightSpec((self.qk_width, s.hidden), stack="qkvg"),
+                "v": WeightSpec((self.v_width, s.hidden), stack="qkvg"), "g": WeightSpec((self.v_width, s.hidden), stack="qkvg"),
+                "o": WeightSpec((s.hidden, self.v_width)), "norm": WeightSpec((self.v_width,), keep_float32=True)}
+
+    def bind(self, weights):
+        import math
+        self.proj = stacked([weights[n] for n in ("q", "k", "v", "g")])
+        self.norm, self.o = weights["norm"], weights["o"]
+        # (the logarithm in 64-bit, rounded once: the kernel's exp gives the decay back to the last bit or so)
+        self._log_decay = torch.tensor([math.log(float(d)) for d in self.spec.decay], dtype=torch.float32,
+                                       device=self.o.device)
+
+    def cache_spec(self):
+        s = self.spec
+        return StateSpec((s.heads * s.head_dim * s.value_dim,), torch.float32)
+
+    def libraries(self):
+        return ["gemm", "recurrence", "elementwise"]
+
+    def workspace_plan(self, rows, dtype, limits):
+        s = self.spec
+        return {("decayed_proj", dtype): rows * (2 * self.qk_width + 2 * self.v_width),
+                ("recurrent_out", torch.float32): rows * self.v_width, ("recurrent_normed", dtype): rows * self.v_width,
+                (self.out_name, dtype): rows * s.hidden, (f"token_groups_{WHOLE}_0", torch.int32): 2 * rows + 2,
+                **_pieces_plan(rows, s.heads * s.head_dim * s.value_dim, s.heads, s.head_dim)}
+
+    def forward(self, ctx, x, cache_id, write_cache=True):
+        s = self.spec
+        k = ctx.kernels
+        m = x.shape[0]
+        ws = ctx.workspace
+        proj = ws.get("decayed_proj", (m, self.proj.shape[0]), x.dtype)
+        k.gemm(x, self.proj, proj)
+        a, b = self.qk_width, 2 * self.qk_width
+        c = b + self.v_width
+        o = ws.get("recurrent_out", (m, self.v_width), torch.float32)
+        _recurrence(ctx, s.heads * s.head_dim * s.value_dim, s.heads, s.head_dim,
+                    proj[:, :a], proj[:, a:b], proj[:, b:c], self._log_decay, o, ctx.cache.state_view(cache_id),
+                    ctx.cache.state_stage(cache_id), 0, ctx.slots, s.heads, s.head_dim, s.value_dim,
+                    write_state=write_cache, activation=s.activation)
+        y = ws.get("recurrent_normed", (m, self.v_width), x.dtype)
+        k.gated_part_norm(o, proj[:, c:], self.norm, y, self.v_width, float(s.eps), gate_first=False, gate_kind=s.gate)
+        out = ws.get(self.out_name, (m, s.hidden), x.dtype)
+        k.gemm(y, self.o, out)
+        return out
+
+
+@register_part("mixer", "delta_rule")
+class DeltaRule:
+    """The gated delta rule with a decay per key channel.  One stacked projection gives q, k (kv_heads x head_dim each)
+    and v (heads x value_dim); q, k, v pass a short causal convolution per
+    channel (no bias) and silu; inside the recurrence kernel q and k become unit vectors per head and q is multiplied
+    by head_dim^(-1/2), beta = sigmoid(Wb x) a head, the decays g = exp(-exp(A_log) softplus(Wa2 (Wa1 x) + dt_bias))
+    per head and key channel; per head S <- diag(g) S, u = beta (v - S^T k), S <- S + k u^T, o = S^T q.  Each head's o
+    is divided by its root mean square over the value channels, multiplied by a weight the heads share and by
+    sigmoid(Wg2 (Wg1 x)), and projected by Wo.  A request's state is S [heads, head_dim, value_dim] and the
+    convolution's last taps - 1 inputs.  Decays, beta, the unit norms and the state are 32-bit."""
+    graph_safe = True
+
+    def __init__(self, spec):
+        s = self.spec = spec
+        if s.heads % s.kv_heads != 0:
+            raise PartError(f"heads {s.heads} is no multiple of kv_heads {s.kv_heads}")
+        if not 1 <= s.head_dim <= 256:
+            raise PartError(f"head_dim {s.head_dim}: the recurrence kernel takes up to 256 key channels a head")
+        if not 1 <= s.conv_taps <= 8:
+            raise PartError(f"conv_taps {s.conv_taps}: the convolution kernel takes 1 to 8 taps")
+        self.qk_width, self.v_width = s.kv_heads * s.head_dim, s.heads * s.value_dim
+        self.decay_width = s.heads * s.head_dim
+        self.channels = 2 * self.qk_width + self.v_width
+        self.state_floats = s.heads * s.head_dim * s.value_dim
+        self.out_name = "mixer_out"
+        self.proj = self.conv = self.beta = self.a1 = self.g1 = self.a2 = self.g2 = None
+        self.dt_bias = self.a_log = self.norm = self.o = None
+        self.decay_rank, self.gate_rank = s.decay_rank or 0, s.gate_rank or 0
+
+    def weight_specs(self):
+        s = self.spec
+        taps = lambda n: WeightSpec((n, s.conv_taps), keep_float32=True, init=("normal", 0.0, 0.4))
+        return {"q": WeightSpec((self.qk_width, s.hidden), stack="in"), "k": WeightSpec((self.qk_width, s.hidden), stack="in"),
+                "v": WeightSpec((self.v_width, s.hidden), stack="in"),
+                "a1": WeightSpec((s.decay_rank, s.hidden)), "g1": WeightSpec((s.gate_rank, s.hidden)),
+                "b": WeightSpec((s.heads, s.hidden)),
+                "q.conv": taps(self.qk_width), "k.conv": taps(self.qk_width), "v.conv": taps(self.v_width),
+                "a2": WeightSpec((self.decay_width, s.decay_rank), init=("normal", 0.0, 0.3)),
+                "dt_bias": WeightSpec((self.decay_width,), keep_float32=True, init=("uniform", -4.0, 0.0)),
+                "A_log": WeightSpec((s.heads,), keep_float32=True, init=("uniform", -1.0, 1.5)),
+                "g2": WeightSpec((self.v_width, s.gate_rank), init=("normal", 0.0, 0.3)),
+                "norm": WeightSpec((s.value_dim,), keep_float32=True), "o": WeightSpec((s.hidden, self.v_width))}
+
+    def bind(self, weights):
+        self.proj = stacked([weights[n] for n in ("q", "k", "v")])
+        self.conv = torch.cat([weights["q.conv"], weights["k.conv"], weights["v.conv"]]).contiguous()
+        self.a1, self.g1, self.beta = weights["a1"], weights["g1"], weights["b"]
+        self.a2, self.g2 = weights["a2"], weights["g2"]
+        self.decay_rank, self.gate_rank = self.a1.shape[0], self.g1.shape[0]
+        if self.a2.shape[1] != self.decay_rank or self.g2.shape[1] != self.gate_rank:
+            raise PartError("the low-rank pairs of the decay or of the gate do not fit each other")
+        self.dt_bias, self.a_log, self.norm, self.o = weights["dt_bias"], weights["A_log"], weights["norm"], weights["o"]
+
+    def cache_spec(self):
+        return StateSpec((self.state_floats + (self.spec.conv_taps - 1) * self.channels,), torch.float32)
+
+    def libraries(self):
+        return ["gemm", "recurrence", "elementwise"]
+
+    def workspace_plan(self, rows, dtype, limits):
+        s = self.spec
+        return {("delta_proj", dtype): rows * self.channels, ("delta_conv", dtype): rows * self.channels,
+                ("delta_low_a", dtype): rows * self.decay_rank, ("delta_low_g", dtype): rows * self.gate_rank,
+                ("delta_z", torch.float32): rows * self.decay_width,
+                ("log_decay", torch.float32): rows * self.decay_width, ("delta_beta", torch.float32): rows * s.heads,
+                ("delta_gate", dtype): rows * self.v_width,
+                ("recurrent_out", torch.float32): rows * self.v_width, ("recurrent_normed", dtype): rows * self.v_width,
+                (self.out_name, dtype): rows * s.hidden, (f"token_groups_{WHOLE}_0", torch.int32): 2 * rows + 2}
+
+    def forward(self, ctx, x, cache_id, write_cache=True):
+        s = self.spec
+        k = ctx.kernels
+        m = x.shape[0]
+        ws = ctx.workspace
+        proj = ws.get("delta_proj", (m, self.proj.shape[0]), x.dtype)
+        k.gemm(x, self.proj, proj)
+        live, stage = ctx.cache.state_view(cache_id), ctx.cache.state_stage(cache_id)
+        conv = ws.get("delta_conv", (m, self.channels), x.dtype)
+        k.causal_conv(proj, self.conv, None, conv, live, stage, self.state_floats, ctx.slots, ctx.positions,
+                      silu=True, write_state=write_cache)
+        # the decays: a low-rank pair whose second product leaves 32-bit sums, then softplus and the head's rate
+        low_a = ws.get("delta_low_a", (m, self.decay_rank), x.dtype)
+        k.gemm(x, self.a1, low_a)
+        z = ws.get("delta_z", (m, self.decay_width), torch.float32)
+        k.gemm(low_a, self.a2, z)
+        log_decay = ws.get("log_decay", (m, self.decay_width), torch.float32)
+        k.channel_log_decay(z, self.dt_bias, self.a_log, log_decay, s.heads, s.head_dim)
+        low_g = ws.get("delta_low_g", (m, self.gate_rank), x.dtype)
+        k.gemm(x, self.g1, low_g)
+        gate = ws.get("delta_gate", (m, self.v_width), x.dtype)
+        k.gemm(low_g, self.g2, gate)
+        beta = ws.get("delta_beta", (m, s.heads), torch.float32)       # (the sigmoid is the recurrence kernel's)
+        k.gemm(x, self.beta, beta)
+        first, count, n = _requests(ctx)
+        a, b = self.qk_width, 2 * self.qk_width
+        o = ws.get("recurrent_out", (m, self.v_width), torch.float32)
+        k.delta_rule(conv[:, :a], conv[:, a:b], conv[:, b:], log_decay, beta, o, live, stage, 0, first, count, n, ctx.slots,
+                     s.heads, s.head_dim, s.value_dim, heads_per_group=s.heads // s.kv_heads,
+                     q_scale=float(s.head_dim) ** -0.5, unit_eps=float(s.unit_eps), write_state=write_cache)
+        y = ws.get("recurrent_normed", (m, self.v_width), x.dtype)
+        k.gated_part_norm(o, gate, self.norm, y, s.value_dim, float(s.eps), gate_first=False, gate_kind="sigmoid")
+        out = ws.get(self.out_name, (m, s.hidden), x.dtype)
+        k.gemm(y, self.o, out)
         return out

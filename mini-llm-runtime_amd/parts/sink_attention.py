@@ -4,15 +4,18 @@ head that stands for no key and brings no value -- and whose queries see the key
 request's first token.
 
 `SinkAttention`: grouped-query attention with query/key and value sizes of their own, optional biases on q, k, v,
-a norm per head of q and k before the rotation, and a rotation of a head's first channels (how many, and the
-angles, are the position part's).  Per token the cache keeps keys [kv_heads, head_dim] and values
-[kv_heads, value_dim], both row-major.
+a norm per head of q and k before the rotation (or after it; with a weight shared by the heads or without one), a
+rotation of a head's first channels (how many, their pairing and the angles are the position part's), and
+optionally a gate on the heads' outputs (sigmoid(Wg x), before the output projection).  Per token the cache keeps
+keys [kv_heads, head_dim] and values [kv_heads, value_dim], both row-major.  The sink may be left out: the usual
+softmax.
 
 `LatentAttention`: keys and values of all heads are up-projections of ONE normed latent vector a token, plus one
 rotated key part that all heads share; only the latent vector and that part are cached, [rank + rot_dim] a token.
 The up-projections are moved to the query's side: q_lat[h] = W_uk[h]^T q_plain[h], so a head's score is
 q_lat[h] . latent + q_rot[h] . k_rot -- attention of all heads over ONE shared key row whose first `rank` channels
-are also the value -- and the head's output is W_uv[h] applied to the attention's latent result.
+are also the value -- and the head's output is W_uv[h] applied to the attention's latent result.  With `q_rank` the
+queries come through a normed latent of their own, q = W_uq norm(W_dq x).
 """
 from __future__ import annotations
 
@@ -32,16 +35,15 @@ def _mask_of(spec):
 
 
 def _rope_table(position, ctx, device, rot_limit):
+    """(the position part's table, whether its pairs are interleaved), or (None, False) without a rotation."""
     if position is None:
-        return None
+        return None, False
     rotation = position.rotation(ctx.max_positions, device)
     if rotation is None:
-        return None
-    if rotation.interleaved or rotation.dim % 2 != 0 or not 2 <= rotation.dim <= rot_limit or \
-            rotation.table.shape[1] != rotation.dim:
-        raise PartError(f"the position part turns {rotation.dim} channels: must be even, in split-half pairs, at most "
-                        f"{rot_limit}")
-    return rotation.table
+        return None, False
+    if rotation.dim % 2 != 0 or not 2 <= rotation.dim <= rot_limit or rotation.table.shape[1] != rotation.dim:
+        raise PartError(f"the position part turns {rotation.dim} channels: must be even, at most {rot_limit}")
+    return rotation.table, bool(rotation.interleaved)
 
 
 PARTIAL_CAP = 8 << 20         # floats that the shares of the key ranges of one launch may take at most
@@ -114,16 +116,22 @@ class SinkAttention:
         self.position = build_part("position", s.position) if s.position is not None else None
         self.q_width, self.k_width, self.v_width = s.q_heads * s.head_dim, s.kv_heads * s.head_dim, s.kv_heads * s.value_dim
         self.o_width = s.q_heads * s.value_dim
+        if s.gate not in (None, "sigmoid", "silu"):
+            raise PartError(f"gate {s.gate!r}: sigmoid, silu or none")
+        self.norm_order = None if s.qk_norm is None else "after" if s.qk_norm_after_rotation else "before"
+        self.out_name = "mixer_out"                      # (a part that runs several mixers gives each a buffer of its own)
         self.qkv = self.o = self.bias = self.q_norm = self.k_norm = self.sink = None
 
     def weight_specs(self):
         s = self.spec
         specs = {"q": WeightSpec((self.q_width, s.hidden), stack="qkv"), "k": WeightSpec((self.k_width, s.hidden), stack="qkv"),
                  "v": WeightSpec((self.v_width, s.hidden), stack="qkv"), "o": WeightSpec((s.hidden, self.o_width))}
+        if s.gate is not None:                           # (behind q, k, v: one projection gives all four)
+            specs["g"] = WeightSpec((self.o_width, s.hidden), stack="qkv")
         if s.bias:
             for name, width in (("q.b", self.q_width), ("k.b", self.k_width), ("v.b", self.v_width)):
                 specs[name] = WeightSpec((width,), keep_float32=True, init=("normal", 0.0, 0.02))
-        if s.qk_norm is not None:
+        if s.qk_norm is not None and s.qk_norm_weight:
             specs["q.norm"] = WeightSpec((s.head_dim,), keep_float32=True)
             specs["k.norm"] = WeightSpec((s.head_dim,), keep_float32=True)
         if s.sink:
@@ -132,10 +140,10 @@ class SinkAttention:
 
     def bind(self, weights):
         s = self.spec
-        self.qkv = stacked([weights["q"], weights["k"], weights["v"]])
+        self.qkv = stacked([weights[n] for n in (("q", "k", "v", "g") if s.gate is not None else ("q", "k", "v"))])
         self.o = weights["o"]
         self.bias = torch.cat([weights["q.b"], weights["k.b"], weights["v.b"]]).contiguous() if s.bias else None
-        if s.qk_norm is not None:
+        if s.qk_norm is not None and s.qk_norm_weight:
             self.q_norm, self.k_norm = weights["q.norm"], weights["k.norm"]
         self.sink = weights["sink"] if s.sink else None
 
@@ -145,12 +153,13 @@ class SinkAttention:
                          self.mask_size if self.mask is not None else None)
 
     def libraries(self):
-        return ["gemm", "sink_attention"]
+        return ["gemm", "sink_attention", "elementwise"]
 
     def workspace_plan(self, rows, dtype, limits):
         s = self.spec
-        return {("sink_proj", dtype): rows * (self.q_width + self.k_width + self.v_width), ("q", dtype): rows * self.q_width,
-                ("attn", dtype): rows * self.o_width, ("mixer_out", dtype): rows * s.hidden,
+        gate = self.o_width if s.gate is not None else 0
+        return {("sink_proj", dtype): rows * (self.q_width + self.k_width + self.v_width + gate), ("q", dtype): rows * self.q_width,
+                ("attn", dtype): rows * self.o_width, (self.out_name, dtype): rows * s.hidden,
                 **_groups_plan(rows, s.q_heads, s.kv_heads, s.value_dim)}
 
     def forward(self, ctx, x, cache_id, write_cache=True):
@@ -162,14 +171,17 @@ class SinkAttention:
         view = ctx.cache.paged_view(cache_id)
         k_pages, v_pages = view.tensors["k"], view.tensors["v"]
         q = ctx.workspace.get("q", (m, self.q_width), x.dtype)
-        rope = _rope_table(self.position, ctx, x.device, s.head_dim)
+        rope, interleaved = _rope_table(self.position, ctx, x.device, s.head_dim)
+        qkv_width = self.q_width + self.k_width + self.v_width
         k.sink_qkv_prep(proj, self.bias, q, k_pages, v_pages, view.block_table, ctx.slots, ctx.positions, self.q_norm,
                         self.k_norm, s.qk_norm.eps if s.qk_norm is not None else 0.0, rope, s.q_heads, s.kv_heads,
-                        s.head_dim, s.value_dim, view.page_size, write_cache)
+                        s.head_dim, s.value_dim, view.page_size, write_cache, norm=self.norm_order, interleaved=interleaved)
         attn = ctx.workspace.get("attn", (m, self.o_width), x.dtype)
         attend(ctx, q, k_pages, v_pages, view, self.sink, attn, s.q_heads, s.kv_heads, s.head_dim, s.value_dim,
                float(s.scale), self.mask, self.mask_size)
-        out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
+        if s.gate is not None:
+            k.gate_mul(attn, proj[:, qkv_width:], attn, s.gate)
+        out = ctx.workspace.get(self.out_name, (m, s.hidden), x.dtype)
         k.gemm(attn, self.o, out)
         return out
 
@@ -187,11 +199,17 @@ class LatentAttention:
         self.q_width = s.heads * (s.head_dim + s.rot_dim)
         self.row = s.rank + s.rot_dim                    # a token's cache row, and a query head after the move
         self.o_width = s.heads * s.value_dim
-        self.proj = self.o = self.norm = self.uk_t = self.uv = self.sink = None
+        self.out_name = "mixer_out"
+        self.proj = self.o = self.norm = self.uk_t = self.uv = self.sink = self.uq = self.q_norm = None
 
     def weight_specs(self):
         s = self.spec
-        specs = {"q": WeightSpec((self.q_width, s.hidden), stack="down"), "dkv": WeightSpec((self.row, s.hidden), stack="down"),
+        if s.q_rank is None:
+            first = {"q": WeightSpec((self.q_width, s.hidden), stack="down")}
+        else:           # the queries' latent comes out of the same projection as the keys' and values'
+            first = {"dq": WeightSpec((s.q_rank, s.hidden), stack="down"), "dq.norm": WeightSpec((s.q_rank,), keep_float32=True),
+                     "uq": WeightSpec((self.q_width, s.q_rank))}
+        specs = {**first, "dkv": WeightSpec((self.row, s.hidden), stack="down"),
                  "dkv.norm": WeightSpec((s.rank,), keep_float32=True),
                  "uk": WeightSpec((s.heads * s.head_dim, s.rank)), "uv": WeightSpec((self.o_width, s.rank)),
                  "o": WeightSpec((s.hidden, self.o_width))}
@@ -201,7 +219,11 @@ class LatentAttention:
 
     def bind(self, weights):
         s = self.spec
-        self.proj = stacked([weights["q"], weights["dkv"]])
+        if s.q_rank is None:
+            self.proj = stacked([weights["q"], weights["dkv"]])
+        else:
+            self.proj = stacked([weights["dq"], weights["dkv"]])
+            self.uq, self.q_norm = weights["uq"], weights["dq.norm"]
         self.norm = weights["dkv.norm"]
         # the key up-projection as the queries meet it: per head [rank, head_dim]
         self.uk_t = weights["uk"].view(s.heads, s.head_dim, s.rank).transpose(1, 2).contiguous()
@@ -213,35 +235,48 @@ class LatentAttention:
         return PagedSpec((("latent", (1, PAGE, self.row)),), self.mask_size if self.mask is not None else None)
 
     def libraries(self):
-        return ["gemm", "grouped_gemm", "sink_attention"]
+        return ["gemm", "grouped_gemm", "sink_attention", "elementwise"]
 
     def workspace_plan(self, rows, dtype, limits):
         s = self.spec
-        return {("latent_proj", dtype): rows * (self.q_width + self.row), ("latent_q", dtype): rows * s.heads * self.row,
+        first = self.q_width if s.q_rank is None else s.q_rank
+        more = {} if s.q_rank is None else {("latent_cq", dtype): rows * s.q_rank, ("latent_queries", dtype): rows * self.q_width}
+        return {("latent_proj", dtype): rows * (first + self.row), ("latent_q", dtype): rows * s.heads * self.row,
                 ("latent_out", dtype): rows * s.heads * s.rank, ("attn", dtype): rows * self.o_width,
-                ("mixer_out", dtype): rows * s.hidden, **_groups_plan(rows, s.heads, 1, s.rank)}
+                (self.out_name, dtype): rows * s.hidden, **more, **_groups_plan(rows, s.heads, 1, s.rank)}
 
     def forward(self, ctx, x, cache_id, write_cache=True):
         s = self.spec
         k = ctx.kernels
         m = x.shape[0]
-        ld = self.q_width + self.row
+        ld = self.proj.shape[0]
         proj = ctx.workspace.get("latent_proj", (m, ld), x.dtype)
         k.gemm(x, self.proj, proj)
         view = ctx.cache.paged_view(cache_id)
         pages = view.tensors["latent"]
         q = ctx.workspace.get("latent_q", (m, s.heads * self.row), x.dtype)
-        rope = _rope_table(self.position, ctx, x.device, s.rot_dim)
-        k.latent_prep(proj, q, pages, view.block_table, ctx.slots, ctx.positions, self.norm, float(s.eps), rope, s.heads,
-                      s.head_dim, s.rot_dim, s.rank, view.page_size, write_cache)
+        rope, interleaved = _rope_table(self.position, ctx, x.device, s.rot_dim)
+        if s.q_rank is None:
+            queries, q_ld = proj, ld
+            k.latent_prep(proj, q, pages, view.block_table, ctx.slots, ctx.positions, self.norm, float(s.eps), rope, s.heads,
+                          s.head_dim, s.rot_dim, s.rank, view.page_size, write_cache, interleaved=interleaved)
+        else:
+            # the queries' latent: normed in 32-bit over its own root mean square, then up to the heads
+            cq = ctx.workspace.get("latent_cq", (m, s.q_rank), x.dtype)
+            k.rmsnorm_columns(proj[:, :s.q_rank], self.q_norm, cq, float(s.eps))
+            queries, q_ld = ctx.workspace.get("latent_queries", (m, self.q_width), x.dtype), self.q_width
+            k.gemm(cq, self.uq, queries)
+            k.latent_prep(proj[:, s.q_rank:], q, pages, view.block_table, ctx.slots, ctx.positions, self.norm, float(s.eps),
+                          rope, s.heads, s.head_dim, s.rot_dim, s.rank, view.page_size, write_cache, q_src=queries,
+                          interleaved=interleaved)
         # the plain query channels through the key up-projection, head by head, into the first `rank` channels
-        k.heads_gemm(torch.as_strided(proj, (m, s.heads, s.head_dim), (ld, s.head_dim + s.rot_dim, 1)), self.uk_t,
+        k.heads_gemm(torch.as_strided(queries, (m, s.heads, s.head_dim), (q_ld, s.head_dim + s.rot_dim, 1)), self.uk_t,
                      torch.as_strided(q, (m, s.heads, s.rank), (s.heads * self.row, self.row, 1)))
         lat = ctx.workspace.get("latent_out", (m, s.heads * s.rank), x.dtype)
         attend(ctx, q, pages, pages, view, self.sink, lat, s.heads, 1, self.row, s.rank, float(s.scale), self.mask,
                self.mask_size)
         attn = ctx.workspace.get("attn", (m, self.o_width), x.dtype)
         k.heads_gemm(lat.view(m, s.heads, s.rank), self.uv, attn.view(m, s.heads, s.value_dim))
-        out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
+        out = ctx.workspace.get(self.out_name, (m, s.hidden), x.dtype)
         k.gemm(attn, self.o, out)
         return out
