@@ -16,7 +16,8 @@ part.
 
 config.json: `architecture` (the name), `vocab`, `width`, `norm.eps`, `embedding.bigram` {`buckets`, `mul_prev`,
 `mul_cur`}, and `layers`, a list of {`type`, `mixer`: sizes and constants, `mlp`: null or {`kind`: dense, `ff`},
-optionally `weights_of`: the layer whose tensors it uses}.  Positions are not bounded by the model; `max_positions`,
+optionally `weights_of`: the layer whose tensors it uses}.  The ranks of the delta rule's low-rank pairs are read off
+the tensors; `mixer.decay_rank` and `mixer.gate_rank` may name them (the random-weights mode needs that).  Positions are not bounded by the model; `max_positions`,
 when a file gives it, bounds what the engine plans for.
 """
 from __future__ import annotations
@@ -82,9 +83,12 @@ def _channel_delta(m, width, eps, where):
     heads, kv = _int(m, "heads", where), _int(m, "kv_heads", where)
     if heads % kv != 0:
         raise ConfigError(f"config.json: {where}heads {heads} is no multiple of kv_heads {kv}")
+    # (the ranks of the two low-rank pairs are the tensors' to say; a configuration may name them, which the
+    # random-weights mode needs)
+    ranks = {key: _int(m, key, where) if m.get(key) is not None else None for key in ("decay_rank", "gate_rank")}
     return DeltaRuleSpec(kind="delta_rule", hidden=width, heads=heads, kv_heads=kv, head_dim=_int(m, "dim", where),
                          value_dim=_int(m, "vdim", where), conv_taps=_int(m, "conv", where), eps=eps,
-                         unit_eps=DELTA_UNIT_EPS)
+                         unit_eps=DELTA_UNIT_EPS, decay_rank=ranks["decay_rank"], gate_rank=ranks["gate_rank"])
 
 
 def _latent_attention(m, width, eps, where):
