@@ -24,6 +24,8 @@ many gigabytes).  Every runner is built with the product's own defaults.  One JS
     feed-forward and layers, with milliseconds per kernel class.  The default workload is not touched by it.
   * --only pamunex: the same for Pamunex models (latent attention over a sliding window beside a dense feed-forward,
     chunked grouped-query attention beside a mixture of experts, in turn).
+  * --only tigelorn: the same for Tigelorn models (windowed attention beside constant-decay linear attention, the
+    gated delta rule, latent attention with a query latent, in turn), beside a Taletar model of equal sizes.
 """
 import argparse
 import json
@@ -558,14 +560,93 @@ class PamunexBench(Bench):
                     frac=round(step_bytes / (seconds / steps) / HBM_PEAK, 5)), step_bytes, report
 
 
+# `--only tigelorn`: layer sizes that resemble a real model's, for a Tigelorn model whose layers take, in turn, windowed
+# attention beside constant-decay linear attention, the gated delta rule, latent attention with a query latent, and the
+# two side by side again, each beside a gated feed-forward (gelu), and for the closest model the engine had before: a
+# Taletar model (Mamba-2, differential attention twice, gated linear attention in turn) of the same width,
+# feed-forward, heads and number of layers.
+TIGELORN_SIZES = {
+    "2k": dict(width=2048, ff=5632, vocab=32000, layers=8, heads=16, kv_heads=4, window=1024, kv_rank=512, q_rank=768,
+               low_rank=64),
+    "4k": dict(width=4096, ff=12288, vocab=32000, layers=8, heads=32, kv_heads=8, window=1024, kv_rank=512, q_rank=1536,
+               low_rank=128),
+}
+
+
+class TigelornBench(Bench):
+    """A Tigelorn model of TIGELORN_SIZES[size] with random weights drawn on the GPU."""
+
+    def __init__(self, size, args):
+        import torch
+        from mini_llm_runtime_amd.api import parse_dtype
+        from mini_llm_runtime_amd.config import config_from_dict
+        from mini_llm_runtime_amd.parts import DecoderModel, expected_tensors
+        from mini_llm_runtime_amd.weights import random_tensors_on_device
+        d = TIGELORN_SIZES[size]
+        self.torch, self.args, self.size = torch, args, size
+        self.dtype = parse_dtype(args.dtype)
+        self.tag = "bf16" if self.dtype == torch.bfloat16 else "fp32"
+        h = d["heads"]
+        left = dict(heads=h, kv_heads=d["kv_heads"], dim=128, vdim=128, scale=128 ** -0.5, rot=dict(dims=64, base=1000000.0),
+                    mask=dict(size=d["window"]))
+        right = dict(heads=h, dim=128, vdim=128, decay=[1.0 - 2.0 ** -(2 + 6 * i / (h - 1)) for i in range(h)])
+        mlp = dict(kind="dense", ff=d["ff"])
+        parallel = dict(type="parallel", mixer=dict(left=left, right=right, left_scale=0.5, right_scale=0.5), mlp=mlp)
+        delta = dict(type="channel_delta", mlp=mlp,
+                     mixer=dict(heads=h, kv_heads=h // 2, dim=128, vdim=128, conv=4, decay_rank=d["low_rank"], gate_rank=d["low_rank"]))
+        latent = dict(type="latent_attention", mlp=mlp,
+                      mixer=dict(heads=h, dim=128, rot_dim=64, vdim=128, kv_rank=d["kv_rank"], q_rank=d["q_rank"], scale=192 ** -0.5,
+                                 rot=dict(dims=64, base=10000.0, scaling=dict(factor=40.0, original=4096, fast=32.0, slow=1.0))))
+        turn = [parallel, delta, latent, parallel]
+        self.layers = self.full_layers = d["layers"]
+        layers = [turn[i % 4] for i in range(self.layers)]
+        kinds = [layer["type"] for layer in layers]
+        self.cfg = config_from_dict(dict(architecture="Tigelorn", vocab=d["vocab"], width=d["width"], norm=dict(eps=1e-5),
+                                         embedding=dict(bigram=dict(buckets=16381, mul_prev=1000003, mul_cur=31)), layers=layers))
+        self.model = DecoderModel(self.cfg, random_tensors_on_device(expected_tensors(self.cfg), 0, self.dtype, "cuda"),
+                                  self.dtype, "cuda:0")
+        self.weights_from = "drawn on the GPU"
+        self.elem = 2 if self.dtype == torch.bfloat16 else 4
+        pair_table = 16382 * d["width"]
+        # (the table is read once, as the head; of the pair table one row a token)
+        self.weight_bytes = self.model.weight_bytes() - pair_table * self.elem
+        self.matrix_params = (self.model.weight_bytes() // self.elem) - d["vocab"] * d["width"] - pair_table
+        n_parallel, n_delta, n_latent = (kinds.count(t) for t in ("parallel", "channel_delta", "latent_attention"))
+        # cache rows that a decoding token's attention reads: keys and values of the kv heads over the window, the latent
+        # row once for all heads over the whole context; recurrent state read and written a step (32-bit)
+        self.window_row_bytes = n_parallel * d["kv_heads"] * 2 * 128 * self.elem
+        self.latent_row_bytes = n_latent * (d["kv_rank"] + 64) * self.elem
+        self.state_bytes = (n_parallel + n_delta) * h * 128 * 128 * 4 * 2
+        self.kv_bytes_per_token = 0                  # (see decode_point)
+        seen = lambda t: sum(min(p, d["window"] - 1) + 1 for p in range(t))
+        self.attention_flops = lambda t: (n_parallel * 2.0 * seen(t) * h * 256 + n_latent * 2.0 * (t * (t + 1) / 2) * h * (2 * d["kv_rank"] + 64)
+                                          + (n_parallel * 2 + n_delta * 3) * 2.0 * t * h * 128 * 128)
+        self.vocab = d["vocab"]
+        self.g = torch.Generator().manual_seed(0)
+
+    def prefill_flops(self, t):
+        d = TIGELORN_SIZES[self.size]
+        return 2.0 * t * self.matrix_params + self.attention_flops(t) + 2.0 * d["vocab"] * d["width"]
+
+    def decode_point(self, batch, steps, warmup, context=None):
+        d = TIGELORN_SIZES[self.size]
+        seconds, mean_context, report = self.decode(batch, steps, warmup, context)
+        step_bytes = self.weight_bytes + batch * (min(mean_context, d["window"]) * self.window_row_bytes
+                                                  + mean_context * self.latent_row_bytes + self.state_bytes)
+        return dict(tok_s=round(batch * steps / seconds, 1), ms=round(seconds / steps * 1e3, 4),
+                    frac=round(step_bytes / (seconds / steps) / HBM_PEAK, 5)), step_bytes, report
+
+
 def design_block(args):
-    """Prefill (2048 tokens in one step) and decode (batch 8 and 64 behind --context tokens) of the Taletar sizes
-    beside a Qwen3 dense model of equal width, heads, feed-forward and layers; then the same steps once more with
-    events around every launch: milliseconds per kernel class."""
+    """Prefill (2048 tokens in one step) and decode (batch 8 and 64 behind --context tokens) of a design's sizes
+    beside the closest model the engine had before it (a Qwen3 dense model of equal width, heads, feed-forward and
+    layers; for Tigelorn a Taletar model of equal sizes); then the same steps once more with events around every
+    launch: milliseconds per kernel class."""
     import copy
     out = {}
     design = getattr(args, "design", "taletar")
-    table, make_design = (PAMUNEX_SIZES, PamunexBench) if design == "pamunex" else (DESIGN_SIZES, TaletarBench)
+    table, make_design = {"pamunex": (PAMUNEX_SIZES, PamunexBench), "tigelorn": (TIGELORN_SIZES, TigelornBench)}.get(
+        design, (DESIGN_SIZES, TaletarBench))
     for size in (args.design_sizes.split(",") if args.design_sizes else list(table)):
         d = table[size]
         dense = (d["layers"], dict(hidden_size=d["width"], num_attention_heads=d["heads"], num_key_value_heads=d["kv_heads"],
@@ -573,7 +654,9 @@ def design_block(args):
                                    max_position_embeddings=40960, rms_norm_eps=1e-6, rope_theta=1000000.0,
                                    tie_word_embeddings=False))
         block = {}
-        for name, make in ((design, lambda a: make_design(size, a)), ("qwen3_dense", lambda a: Bench(size, 0, a, sizes=dense))):
+        beside = ("taletar", lambda a: TaletarBench(size, a)) if design == "tigelorn" else \
+            ("qwen3_dense", lambda a: Bench(size, 0, a, sizes=dense))
+        for name, make in ((design, lambda a: make_design(size, a)), beside):
             plain_args, profiled = copy.copy(args), copy.copy(args)
             plain_args.profile, plain_args.weights = False, "gpu"
             profiled.profile, profiled.weights, profiled.prefill_reps = True, "gpu", 3
@@ -614,12 +697,12 @@ def main():
                          "tensors drawn on the GPU; auto: folder for the 0.6B sizes, gpu for the larger ones")
     ap.add_argument("--warm-up", type=int, default=0,
                     help="--only engine: 1 captures the decoding steps (Engine.warm_up) before the first burst")
-    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "prompt", "engine", "mixed", "taletar", "pamunex"],
+    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "prompt", "engine", "mixed", "taletar", "pamunex", "tigelorn"],
                     help="profiling aid: run just the decode steps, just the prefill or just the mixed step; prompt: one "
                          "prompt of --context tokens in portions of 2048; engine: the "
                          "scheduler over a burst of requests (3 x batch requests of 512 prompt and 128 output tokens, "
                          "batch slots), printed as one line of its own")
-    ap.add_argument("--design-sizes", default="", help="--only taletar / pamunex: which of its sizes (2k, 4k; default both)")
+    ap.add_argument("--design-sizes", default="", help="--only taletar / pamunex / tigelorn: which of its sizes (2k, 4k; default both)")
     ap.add_argument("--library", type=int, default=1,
                     help="0: every matrix product on the hand-written kernels, none in the vendor library")
     ap.add_argument("--split-keys", type=int, default=256, help="the smallest range of keys of one attention workgroup")
@@ -643,7 +726,7 @@ def main():
     if not args.tune:
         from mini_llm_runtime_amd.kernels import build
         build.load("library_gemm").mlr_library_gemm_tuning(0)
-    if args.only in ("taletar", "pamunex"):
+    if args.only in ("taletar", "pamunex", "tigelorn"):
         args.design = args.only
         print(json.dumps({f"{args.only}_sizes": design_block(args), "context": args.context, "dtype": args.dtype}))
         return 0

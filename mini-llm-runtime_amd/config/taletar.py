@@ -22,10 +22,10 @@ DEFAULT_MAX_POSITIONS = 1 << 20
 _LIMIT = 1_000_000
 
 
-def _int(d, key, where, lo=1):
+def _int(d, key, where, lo=1, hi=_LIMIT):
     v = d.get(key)
-    if isinstance(v, bool) or not isinstance(v, int) or not lo <= v <= _LIMIT:
-        raise ConfigError(f"config.json: {where}`{key}` must be an integer in {lo}..{_LIMIT}, got {v!r}")
+    if isinstance(v, bool) or not isinstance(v, int) or not lo <= v <= hi:
+        raise ConfigError(f"config.json: {where}`{key}` must be an integer in {lo}..{hi}, got {v!r}")
     return v
 
 

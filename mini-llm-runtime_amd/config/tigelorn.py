@@ -31,6 +31,7 @@ from .specs import (DecayedLinearAttentionSpec, DeltaRuleSpec, FrequencyStretch,
                     MixerSumSpec, MlpSpec, ModelSpec, NormSpec, PairEmbedSpec, PositionSpec, SinkAttentionSpec)
 from .taletar import DEFAULT_MAX_POSITIONS, _freeze, _int, _num, _thaw
 
+PAIR_LIMIT = (1 << 31) - 2     # buckets of the pair table: its rows are counted in 32 bits
 DELTA_UNIT_EPS = 1e-6          # inside the root that makes q and k of the delta rule unit vectors
 
 
@@ -166,8 +167,8 @@ class TigelornConfig:
         eos_ids = () if eos is None else (eos,) if isinstance(eos, int) else tuple(eos)
         at = "embedding.bigram."
         return cls(vocab=_int(data, "vocab", ""), width=width, eps=_num(data["norm"], "eps", "norm.", positive=True),
-                   buckets=_int(bigram, "buckets", at), mul_prev=_int(bigram, "mul_prev", at, lo=0),
-                   mul_cur=_int(bigram, "mul_cur", at, lo=0), layers=_freeze(layers),
+                   buckets=_int(bigram, "buckets", at, hi=PAIR_LIMIT), mul_prev=_int(bigram, "mul_prev", at, lo=0, hi=1 << 62),
+                   mul_cur=_int(bigram, "mul_cur", at, lo=0, hi=1 << 62), layers=_freeze(layers),
                    max_positions=_int(data, "max_positions", "") if "max_positions" in data else DEFAULT_MAX_POSITIONS,
                    eos_token_ids=eos_ids)
 

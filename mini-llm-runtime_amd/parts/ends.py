@@ -80,8 +80,8 @@ class PairEmbedding(TokenEmbedding):
         h = ctx.workspace.get("hidden", (ctx.n_tokens, s.hidden), torch.float32)
         ctx.kernels.pair_embed(ctx.token_ids, ctx.positions, ctx.slots, self.weight, self.pairs,
                                ctx.cache.state_view(self.cache_id), ctx.cache.state_stage(self.cache_id), h,
-                               s.buckets, s.mul_prev, s.mul_cur)
-        return h
+                               s.buckets, s.mul_prev % s.buckets, s.mul_cur % s.buckets)     # (the same rows; the kernel's
+        return h                                                                                    # products stay small)
 
 
 @register_part("head", "linear_head")
