@@ -369,6 +369,227 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(DeltaArgs a) {
     }
 }
 
+
+// ---- the delta rule over chunks of tokens --------------------------------------------------------------------
+// A request's rows are cut into chunks of at most DC tokens.  With c_t[i] the sum of a chunk's log decays of key
+// channel i up to and including token t, and S0 the state the chunk starts from, the rule's writes u_t obey
+//     u_t = beta_t (v_t - S0^T (k_t e^{c_t}) - sum_{s<t} (sum_i k_t[i] k_s[i] e^{c_t[i] - c_s[i]}) u_s),
+// a unit lower-triangular system (I + A) U = beta (V - Khat S0) whose inverse T depends on the chunk's keys, decays
+// and beta alone.  The first kernel (one workgroup per chunk and head, all side by side) leaves in scratch memory
+//     W = T (beta Khat) [DC, N],  Y = T (beta V) [DC, V],  B[t, s] = sum_i q_t[i] k_s[i] e^{c_t[i] - c_s[i]} (s <= t),
+//     Qhat[t] = q_t e^{c_t},  Kbar[s] = k_s e^{c_last - c_s},  G = e^{c_last};
+// the second (one workgroup per request, head and DELTA_CHUNK_COLS value channels) walks a request's chunks in
+// their order with the state in LDS:  U = Y - W S0;  O = Qhat S0 + B U;  S <- diag(G) S0 + Kbar^T U.
+// Every exponent is a difference c_t - c_s with s <= t or c_t itself, so nothing overflows however strong a decay
+// is.  The result differs from the token-by-token kernel's by 32-bit rounding.
+#define DELTA_CHUNK 32
+#define DELTA_CHUNK_COLS 32
+
+struct DeltaChunkArgs {
+    DeltaArgs d;
+    const int32_t* chunk_first; const int32_t* chunk_count;     // the chunks, a request's one after the other
+    float* scratch;                                              // [chunks][heads][delta_chunk_floats(N, V)]
+};
+
+__host__ __device__ inline size_t delta_chunk_floats(int N, int V) {
+    return (size_t)DELTA_CHUNK * (3 * N + V + DELTA_CHUNK) + N;
+}
+
+__global__ __launch_bounds__(256) void delta_chunk_prepare_kernel(DeltaChunkArgs g) {
+    constexpr int C = DELTA_CHUNK, CS = DELTA_CHUNK + 1;
+    const DeltaArgs& a = g.d;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int N = a.N, V = a.V, NS = N + 1;
+    float* q_l = lds;                    // [C][NS]
+    float* k_l = q_l + C * NS;
+    float* c_l = k_l + C * NS;
+    float* A_l = c_l + C * NS;           // [C][CS]
+    float* B_l = A_l + C * CS;
+    float* T_l = B_l + C * CS;
+    float* beta_l = T_l + C * CS;        // [C]
+    const int chunk = blockIdx.x, head = blockIdx.y;
+    const int r0 = g.chunk_first[chunk], n = g.chunk_count[chunk];
+    const int qk_head = head / a.heads_per_group;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    float* base = g.scratch + ((size_t)chunk * a.heads + head) * delta_chunk_floats(N, V);
+    float* W = base;
+    float* Qh = W + (size_t)C * N;
+    float* Kb = Qh + (size_t)C * N;
+    float* Y = Kb + (size_t)C * N;
+    float* B = Y + (size_t)C * V;
+    float* G = B + C * C;
+    for (int idx = tid; idx < C * N; idx += 256) {
+        const int t = idx / N, i = idx % N;
+        float dq = 0.f, dk = 0.f, dc = 0.f;
+        if (t < n) {
+            const size_t row = (size_t)(r0 + t);
+            dq = to_float(a.q[row * a.q_stride + qk_head * N + i]);
+            dk = to_float(a.k[row * a.k_stride + qk_head * N + i]);
+            dc = a.log_decay[row * ((size_t)a.heads * N) + head * N + i];
+        }
+        q_l[t * NS + i] = dq; k_l[t * NS + i] = dk; c_l[t * NS + i] = dc;
+    }
+    __syncthreads();
+    for (int t = wave; t < C; t += 4) {                     // unit vectors, q scaled; beta
+        float qq = 0.f, kk = 0.f;
+        for (int i = lane; i < N; i += 64) {
+            const float dq = q_l[t * NS + i], dk = k_l[t * NS + i];
+            qq += dq * dq;
+            kk += dk * dk;
+        }
+        float fq = a.q_scale, fk = 1.0f;
+        if (a.unit_norm) {
+            fq = a.q_scale / sqrtf(wave_sum(qq) + a.unit_eps);
+            fk = 1.0f / sqrtf(wave_sum(kk) + a.unit_eps);
+        }
+        for (int i = lane; i < N; i += 64) { q_l[t * NS + i] *= fq; k_l[t * NS + i] *= fk; }
+        if (lane == 0) beta_l[t] = t < n ? sigmoid_f(a.beta_raw[(size_t)(r0 + t) * a.beta_stride + head]) : 0.f;
+    }
+    for (int i = tid; i < N; i += 256) {                    // c_t: the running sum of the log decays (rows past n add 0)
+        float sum = 0.f;
+        for (int t = 0; t < C; ++t) { sum += c_l[t * NS + i]; c_l[t * NS + i] = sum; }
+    }
+    __syncthreads();
+    for (int p = tid; p < C * C; p += 256) {
+        const int t = p / C, s = p % C;
+        float sa = 0.f, sb = 0.f;
+        if (s <= t && t < n) {
+            const float* ct = c_l + t * NS; const float* cs = c_l + s * NS;
+            const float* kt = k_l + t * NS; const float* ks = k_l + s * NS; const float* qt = q_l + t * NS;
+            for (int i = 0; i < N; ++i) {
+                const float x = ks[i] * expf(ct[i] - cs[i]);
+                sa += kt[i] * x;
+                sb += qt[i] * x;
+            }
+        }
+        A_l[t * CS + s] = s < t ? beta_l[t] * sa : 0.f;
+        B_l[t * CS + s] = sb;
+        B[t * C + s] = sb;
+    }
+    for (int idx = tid; idx < C * N; idx += 256) {          // Qhat, Kbar, G (they read what the loop above reads)
+        const int t = idx / N, i = idx % N;
+        const float ct = c_l[t * NS + i], last = c_l[(C - 1) * NS + i];
+        Qh[idx] = q_l[t * NS + i] * expf(ct);
+        Kb[idx] = k_l[t * NS + i] * expf(last - ct);
+        if (t == 0) G[i] = expf(last);
+    }
+    __syncthreads();
+    if (tid < C) {                                          // T = (I + A)^-1, a column a lane, row after row
+        const int j = tid;
+        for (int t = 0; t < C; ++t) {
+            float x = t == j ? 1.f : 0.f;
+            for (int s = 0; s < t; ++s) x -= A_l[t * CS + s] * T_l[s * CS + j];
+            T_l[t * CS + j] = x;
+        }
+    }
+    for (int idx = tid; idx < C * N; idx += 256) {          // beta Khat in q's place
+        const int t = idx / N, i = idx % N;
+        q_l[t * NS + i] = beta_l[t] * k_l[t * NS + i] * expf(c_l[t * NS + i]);
+    }
+    __syncthreads();
+    for (int idx = tid; idx < C * N; idx += 256) {
+        const int t = idx / N, i = idx % N;
+        float acc = 0.f;
+        for (int s = 0; s <= t; ++s) acc += T_l[t * CS + s] * q_l[s * NS + i];
+        W[idx] = acc;
+    }
+    for (int idx = tid; idx < C * V; idx += 256) {
+        const int t = idx / V, j = idx % V;
+        float acc = 0.f;
+        const int last = min(t, n - 1);
+        for (int s = 0; s <= last; ++s)
+            acc += T_l[t * CS + s] * beta_l[s] * to_float(a.v[(size_t)(r0 + s) * a.v_stride + head * V + j]);
+        Y[idx] = acc;
+    }
+}
+
+__global__ __launch_bounds__(256) void delta_chunk_scan_kernel(DeltaChunkArgs g) {
+    constexpr int C = DELTA_CHUNK, CS = DELTA_CHUNK + 1, COLS = DELTA_CHUNK_COLS;
+    const DeltaArgs& a = g.d;
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    const int N = a.N, V = a.V, NS = N + 1;
+    float* S_l = lds;                    // [N][COLS]
+    float* U_l = S_l + N * COLS;         // [C][COLS]
+    float* buf = U_l + C * COLS;         // [C][NS]: W, then Qhat, then Kbar
+    float* B_l = buf + C * NS;           // [C][CS]
+    float* G_l = B_l + C * CS;           // [N]
+    const int seg = blockIdx.x, head = blockIdx.y, col0 = blockIdx.z * COLS;
+    const int r0 = a.seg_first[seg], n = a.seg_count[seg];
+    const int slot = a.slots[r0];
+    const int tid = threadIdx.x, t = tid >> 3, jq = (tid & 7) * 4;
+    int chunk0 = 0;
+    for (int s = 0; s < seg; ++s) chunk0 += (a.seg_count[s] + C - 1) / C;
+    const size_t per = delta_chunk_floats(N, V);
+    const size_t state_at = (size_t)slot * a.state_stride + (size_t)head * N * V;
+    for (int idx = tid; idx < N * COLS; idx += 256) {
+        const int i = idx / COLS, c = col0 + idx % COLS;
+        S_l[idx] = c < V ? a.live[state_at + (size_t)i * V + c] : 0.f;
+    }
+    for (int c0 = 0, chunk = chunk0; c0 < n; c0 += C, ++chunk) {
+        const int nt = min(C, n - c0);
+        const float* base = g.scratch + ((size_t)chunk * a.heads + head) * per;
+        const float* W = base;
+        const float* Qh = W + (size_t)C * N;
+        const float* Kb = Qh + (size_t)C * N;
+        const float* Y = Kb + (size_t)C * N;
+        const float* B = Y + (size_t)C * V;
+        const float* G = B + C * C;
+        __syncthreads();                                    // the state is whole, the chunk before has been read
+        for (int idx = tid; idx < C * N; idx += 256) buf[(idx / N) * NS + idx % N] = W[idx];
+        for (int idx = tid; idx < C * C; idx += 256) B_l[(idx / C) * CS + idx % C] = B[idx];
+        for (int i = tid; i < N; i += 256) G_l[i] = G[i];
+        __syncthreads();
+        float u[4], o[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) u[e] = col0 + jq + e < V ? Y[(size_t)t * V + col0 + jq + e] : 0.f;
+        for (int i = 0; i < N; ++i) {
+            const float w = buf[t * NS + i];
+            const float4 s4 = *reinterpret_cast<const float4*>(S_l + i * COLS + jq);
+            u[0] -= w * s4.x; u[1] -= w * s4.y; u[2] -= w * s4.z; u[3] -= w * s4.w;
+        }
+        *reinterpret_cast<float4*>(U_l + t * COLS + jq) = make_float4(u[0], u[1], u[2], u[3]);
+        __syncthreads();
+        for (int idx = tid; idx < C * N; idx += 256) buf[(idx / N) * NS + idx % N] = Qh[idx];
+        __syncthreads();
+        o[0] = o[1] = o[2] = o[3] = 0.f;
+        for (int i = 0; i < N; ++i) {
+            const float w = buf[t * NS + i];
+            const float4 s4 = *reinterpret_cast<const float4*>(S_l + i * COLS + jq);
+            o[0] += w * s4.x; o[1] += w * s4.y; o[2] += w * s4.z; o[3] += w * s4.w;
+        }
+        for (int s = 0; s <= t; ++s) {
+            const float w = B_l[t * CS + s];
+            const float4 u4 = *reinterpret_cast<const float4*>(U_l + s * COLS + jq);
+            o[0] += w * u4.x; o[1] += w * u4.y; o[2] += w * u4.z; o[3] += w * u4.w;
+        }
+        if (t < nt) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (col0 + jq + e < V) a.out[(size_t)(r0 + c0 + t) * ((size_t)a.heads * V) + head * V + col0 + jq + e] = o[e];
+        }
+        __syncthreads();
+        for (int idx = tid; idx < C * N; idx += 256) buf[(idx / N) * NS + idx % N] = Kb[idx];
+        __syncthreads();
+        for (int i = t; i < N; i += C) {                   // (a thread's own elements of S: no other thread reads them now)
+            float4 s4 = *reinterpret_cast<const float4*>(S_l + i * COLS + jq);
+            const float gi = G_l[i];
+            s4.x *= gi; s4.y *= gi; s4.z *= gi; s4.w *= gi;
+            for (int s = 0; s < C; ++s) {
+                const float w = buf[s * NS + i];
+                const float4 u4 = *reinterpret_cast<const float4*>(U_l + s * COLS + jq);
+                s4.x += w * u4.x; s4.y += w * u4.y; s4.z += w * u4.z; s4.w += w * u4.w;
+            }
+            *reinterpret_cast<float4*>(S_l + i * COLS + jq) = s4;
+        }
+    }
+    __syncthreads();
+    if (a.write_state)
+        for (int idx = tid; idx < N * COLS; idx += 256) {
+            const int i = idx / COLS, c = col0 + idx % COLS;
+            if (c < V) a.stage[state_at + (size_t)i * V + c] = S_l[idx];
+        }
+}
+
 template <int NR, int PARTS>
 static int launch_delta(const DeltaArgs& a, int segments, hipStream_t stream) {
     constexpr int COLS = 64 / PARTS;
@@ -489,6 +710,37 @@ int mlr_delta_rule(const void* q, long q_stride, const void* k, long k_stride, c
     MLR_DELTA(4)
 #undef MLR_DELTA
     return -1;
+}
+
+// The delta rule in chunks (see delta_chunk_prepare_kernel): `chunk_first`/`chunk_count` name the step's chunks of at
+// most DELTA_CHUNK tokens, a request's chunks one after the other and the requests in the order of `seg_first`;
+// scratch: chunks * heads * mlr_delta_chunk_floats(n_keys, n_values) floats.  Up to 128 key channels a head.
+long mlr_delta_chunk_floats(int n_keys, int n_values) { return (long)delta_chunk_floats(n_keys, n_values); }
+int mlr_delta_chunk_tokens() { return DELTA_CHUNK; }
+
+int mlr_delta_rule_chunked(const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
+                           const float* log_decay, const float* beta_raw, long beta_stride, float* out, const float* live,
+                           float* stage, long state_stride, const int32_t* seg_first, const int32_t* seg_count,
+                           const int32_t* slots, int segments, const int32_t* chunk_first, const int32_t* chunk_count, int chunks,
+                           float* scratch, int heads, int heads_per_group, int n_keys, int n_values, int write_state,
+                           int unit_norm, float q_scale, float unit_eps, hipStream_t stream) {
+    if (segments <= 0 || chunks <= 0) return 0;
+    if (n_keys < 1 || n_keys > 128 || n_values < 1 || heads < 1 || heads > 65535 || heads_per_group < 1 ||
+        heads % heads_per_group || scratch == nullptr)
+        return -1;
+    DeltaChunkArgs g{{(const elem_t*)q, q_stride, (const elem_t*)k, k_stride, (const elem_t*)v, v_stride, log_decay, beta_raw,
+                      beta_stride, out, live, stage, state_stride, seg_first, seg_count, slots, heads, heads_per_group, n_keys,
+                      n_values, write_state, unit_norm, q_scale, unit_eps},
+                     chunk_first, chunk_count, scratch};
+    const int C = DELTA_CHUNK, NS = n_keys + 1;
+    const size_t lds1 = sizeof(float) * ((size_t)3 * C * NS + (size_t)3 * C * (C + 1) + C);
+    delta_chunk_prepare_kernel<<<dim3(chunks, heads), 256, lds1, stream>>>(g);
+    int err = (int)hipGetLastError();
+    if (err != 0) return err;
+    const size_t lds2 = sizeof(float) * ((size_t)n_keys * DELTA_CHUNK_COLS + (size_t)C * DELTA_CHUNK_COLS + (size_t)C * NS +
+                                         (size_t)C * (C + 1) + n_keys);
+    delta_chunk_scan_kernel<<<dim3(segments, heads, (n_values + DELTA_CHUNK_COLS - 1) / DELTA_CHUNK_COLS), 256, lds2, stream>>>(g);
+    return (int)hipGetLastError();
 }
 
 }  // extern "C"

@@ -78,7 +78,7 @@ class Runner:
         self.max_logits_rows = min(max_logits_rows or self.max_batch_tokens, self.max_batch_tokens)
         # the memory plan, and the budget gate before anything of it is allocated
         limits = dict(max_length=self.max_length, page_size=page_size, split_keys=split_keys,
-                      split_max_tokens=split_max_tokens, target_workgroups=target_workgroups)
+                      split_max_tokens=split_max_tokens, target_workgroups=target_workgroups, max_slots=max_slots)
         workspace_plan = model.workspace_plan(self.max_batch_tokens, self.max_logits_rows, limits)
         uses_library = library_gemm and self.dtype == torch.bfloat16
         if _kv_dtype(kv_dtype, self.dtype) != self.dtype:

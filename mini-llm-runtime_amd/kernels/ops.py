@@ -967,6 +967,55 @@ class Kernels:
             _c_int(n_values), _c_int(1 if write_state else 0), _c_int(1 if unit_norm else 0), _c_float(q_scale),
             _c_float(unit_eps), _stream()), "delta_rule")
 
+    DELTA_CHUNK_MAX_KEYS = 128
+
+    def delta_chunk_tokens(self):
+        """Tokens in a chunk of `delta_rule_chunked`."""
+        return int(self._lib("recurrence").mlr_delta_chunk_tokens())
+
+    def delta_chunk_floats(self, chunks, heads, n_keys, n_values):
+        """Floats of scratch memory that `delta_rule_chunked` needs for so many chunks."""
+        fn = self._lib("recurrence").mlr_delta_chunk_floats
+        fn.restype = ctypes.c_long
+        return int(chunks) * int(heads) * int(fn(_c_int(n_keys), _c_int(n_values)))
+
+    @timed("recurrence", _tensors_work())
+    def delta_rule_chunked(self, q, k, v, log_decay, beta_raw, out, live, stage, state_offset, seg_first, seg_count, segments,
+                           slots, chunk_first, chunk_count, chunks, scratch, heads, n_keys, n_values, heads_per_group=1,
+                           q_scale=1.0, unit_norm=True, unit_eps=1e-6, write_state=True):
+        """`delta_rule` over chunks of tokens: `chunk_first`/`chunk_count` cut every request of the step into chunks of
+        at most `delta_chunk_tokens()` tokens (a request's chunks one after the other, the requests in the order of
+        `seg_first`); what a chunk does to ANY state it might start from is worked out for all chunks side by side,
+        then a request's chunks are applied in their order.  Up to DELTA_CHUNK_MAX_KEYS key channels a head; the
+        result differs from the token-by-token order by 32-bit rounding."""
+        rows = v.shape[0]
+        _need(heads >= 1 and heads_per_group >= 1 and heads % heads_per_group == 0, "delta_rule_chunked: heads and groups")
+        groups = heads // heads_per_group
+        _need(1 <= n_keys <= self.DELTA_CHUNK_MAX_KEYS, f"delta_rule_chunked: 1..{self.DELTA_CHUNK_MAX_KEYS} key channels a head")
+        qs = self._columns(q, "q", self.dtype, rows, groups * n_keys)
+        ks = self._columns(k, "k", self.dtype, rows, groups * n_keys)
+        vs = self._columns(v, "v", self.dtype, rows, heads * n_values)
+        _tensor(log_decay, "log_decay", torch.float32, (rows, heads * n_keys))
+        bs = self._columns(beta_raw, "beta_raw", torch.float32, rows, heads)
+        _tensor(out, "out", torch.float32, (rows, heads * n_values))
+        self._check_state(live, stage, state_offset, heads * n_keys * n_values)
+        _tensor(seg_first, "seg_first", torch.int32, (segments,))
+        _tensor(seg_count, "seg_count", torch.int32, (segments,))
+        _tensor(chunk_first, "chunk_first", torch.int32, (chunks,))
+        _tensor(chunk_count, "chunk_count", torch.int32, (chunks,))
+        _tensor(slots, "slots", torch.int32, (rows,))
+        _tensor(scratch, "scratch", torch.float32, ndim=1)
+        _need(scratch.numel() >= self.delta_chunk_floats(chunks, heads, n_keys, n_values), "delta_rule_chunked: scratch too small")
+        _need(segments <= 65535 * 32 and heads <= 65535 and chunks >= segments, "delta_rule_chunked: requests, chunks or heads")
+        at = state_offset * 4
+        _ok(self._lib("recurrence").mlr_delta_rule_chunked(
+            _p(q), ctypes.c_long(qs), _p(k), ctypes.c_long(ks), _p(v), ctypes.c_long(vs), _p(log_decay), _p(beta_raw),
+            ctypes.c_long(bs), _p(out), _ptr(live.data_ptr() + at), _ptr(stage.data_ptr() + at), ctypes.c_long(live.stride(0)),
+            _p(seg_first), _p(seg_count), _p(slots), _c_int(segments), _p(chunk_first), _p(chunk_count), _c_int(chunks),
+            _p(scratch), _c_int(heads), _c_int(heads_per_group), _c_int(n_keys), _c_int(n_values),
+            _c_int(1 if write_state else 0), _c_int(1 if unit_norm else 0), _c_float(q_scale), _c_float(unit_eps), _stream()),
+            "delta_rule_chunked")
+
     # -- differential attention -----------------------------------------------------------------------
     DIFF_MAX_HEAD_DIM = 256
     DIFF_MAX_VALUE_DIM = 256

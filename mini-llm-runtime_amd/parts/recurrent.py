@@ -19,6 +19,9 @@ WHOLE = 1 << 30          # `StepContext.token_groups(WHOLE)`: every request of t
 PIECE = 128              # tokens of a piece when a step's portions run in pieces side by side
 PIECES_FROM = 512        # rows of a step from which they do (the bfloat16 engine)
 PIECE_FLOATS = 64 << 20  # floats that the pieces' states may take; a step with more runs token by token
+DELTA_CHUNK = 32         # tokens of a chunk of the delta rule (the kernel's `delta_chunk_tokens()`)
+CHUNKS_FROM = 64         # rows of a step from which the delta rule runs in chunks (the bfloat16 engine), where the
+                         # step's requests bring eight tokens each or more (single tokens stay with the walk)
 
 
 def _requests(ctx):
@@ -346,7 +349,19 @@ class DeltaRule:
                 ("log_decay", torch.float32): rows * self.decay_width, ("delta_beta", torch.float32): rows * s.heads,
                 ("delta_gate", dtype): rows * self.v_width,
                 ("recurrent_out", torch.float32): rows * self.v_width, ("recurrent_normed", dtype): rows * self.v_width,
-                (self.out_name, dtype): rows * s.hidden, (f"token_groups_{WHOLE}_0", torch.int32): 2 * rows + 2}
+                (self.out_name, dtype): rows * s.hidden, (f"token_groups_{WHOLE}_0", torch.int32): 2 * rows + 2,
+                **self._chunks_plan(rows, dtype, limits)}
+
+    def _chunks_plan(self, rows, dtype, limits):
+        """Scratch memory of the chunked rule for a step of at most `rows` tokens: every request of the step may add a
+        ragged chunk."""
+        s = self.spec
+        if dtype != torch.bfloat16 or rows < CHUNKS_FROM or s.head_dim > 128:
+            return {}
+        per = DELTA_CHUNK * (3 * s.head_dim + s.value_dim + DELTA_CHUNK) + s.head_dim      # (`Kernels.delta_chunk_floats`)
+        chunks = rows // DELTA_CHUNK + min(rows, int((limits or {}).get("max_slots") or rows))
+        return {("delta_chunks", torch.float32): min(chunks, max(1, PIECE_FLOATS // (per * s.heads))) * per * s.heads,
+                (f"token_groups_{DELTA_CHUNK}_0", torch.int32): 2 * chunks + 2}
 
     def forward(self, ctx, x, cache_id, write_cache=True):
         s = self.spec
@@ -375,9 +390,20 @@ class DeltaRule:
         first, count, n = _requests(ctx)
         a, b = self.qk_width, 2 * self.qk_width
         o = ws.get("recurrent_out", (m, self.v_width), torch.float32)
-        k.delta_rule(conv[:, :a], conv[:, a:b], conv[:, b:], log_decay, beta, o, live, stage, 0, first, count, n, ctx.slots,
-                     s.heads, s.head_dim, s.value_dim, heads_per_group=s.heads // s.kv_heads,
-                     q_scale=float(s.head_dim) ** -0.5, unit_eps=float(s.unit_eps), write_state=write_cache)
+        more = dict(heads_per_group=s.heads // s.kv_heads, q_scale=float(s.head_dim) ** -0.5, unit_eps=float(s.unit_eps),
+                    write_state=write_cache)
+        chunks_most = m // DELTA_CHUNK + len(ctx.segments)
+        if ctx.dtype == torch.bfloat16 and m >= max(CHUNKS_FROM, 8 * len(ctx.segments)) and s.head_dim <= k.DELTA_CHUNK_MAX_KEYS and \
+                k.delta_chunk_floats(chunks_most, s.heads, s.head_dim, s.value_dim) <= PIECE_FLOATS:
+            # many rows (prompt portions): what a chunk of tokens does to its state for all chunks side by side, then
+            # a request's chunks in their order; the float engine stays with one order of sums a token
+            (c_first, c_count, c_n), _, _ = ctx.token_groups(DELTA_CHUNK, 0)
+            scratch = ws.get("delta_chunks", (k.delta_chunk_floats(c_n, s.heads, s.head_dim, s.value_dim),), torch.float32)
+            k.delta_rule_chunked(conv[:, :a], conv[:, a:b], conv[:, b:], log_decay, beta, o, live, stage, 0, first, count, n,
+                                 ctx.slots, c_first, c_count, c_n, scratch, s.heads, s.head_dim, s.value_dim, **more)
+        else:
+            k.delta_rule(conv[:, :a], conv[:, a:b], conv[:, b:], log_decay, beta, o, live, stage, 0, first, count, n, ctx.slots,
+                         s.heads, s.head_dim, s.value_dim, **more)
         y = ws.get("recurrent_normed", (m, self.v_width), x.dtype)
         k.gated_part_norm(o, gate, self.norm, y, s.value_dim, float(s.eps), gate_first=False, gate_kind="sigmoid")
         out = ws.get(self.out_name, (m, s.hidden), x.dtype)

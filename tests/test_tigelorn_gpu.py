@@ -268,6 +268,69 @@ def test_delta_rule_carries_its_state_across_steps(dtype_name, heads, per_group,
         np.testing.assert_allclose(np.concatenate(got[s]), want[s], atol=3e-5 * scale, rtol=3e-5)
 
 
+@pytest.mark.parametrize("dtype_name", DTYPES)
+@pytest.mark.parametrize("heads,per_group,keys,values", [(2, 1, 24, 40), (4, 2, 16, 24), (1, 1, 1, 1), (1, 1, 70, 65), (2, 2, 128, 100),
+                                                         (2, 1, 33, 64), (4, 1, 64, 32)])
+def test_delta_rule_in_chunks_of_tokens(dtype_name, heads, per_group, keys, values):
+    """Three requests of 150, 1 and 37 tokens in one step, from states that are not zero, cut into chunks of the
+    kernel's size; decays from none at all to e^-30 a token (no quotient of decays may be formed); outputs and staged
+    states against the plain rule continued from the same states."""
+    from mini_llm_runtime_amd.kernels import Kernels
+    dtype = DTYPES[dtype_name]
+    k = Kernels(dtype)
+    rng = np.random.default_rng(keys + values)
+    groups = heads // per_group
+    lengths, slot_of = [150, 1, 37], [2, 0, 3]
+    n = sum(lengths)
+    q, kk = rounded(rng.normal(size=(n, groups * keys)), dtype), rounded(rng.normal(size=(n, groups * keys)), dtype)
+    v = rounded(rng.normal(size=(n, heads * values)), dtype)
+    decay = -np.exp(rng.uniform(-9.0, 3.4, size=(n, heads * keys)))
+    decay[rng.random(size=decay.shape) < 0.1] = 0.0
+    decay = torch.from_numpy(decay).float().cuda()
+    beta = torch.from_numpy(rng.normal(size=(n, heads)) * 2.0).float().cuda()
+    state = heads * keys * values
+    live = torch.from_numpy(rng.normal(size=(4, state))).float().cuda()
+    stage = torch.zeros_like(live)
+    size = k.delta_chunk_tokens()
+    first, count, c_first, c_count, slots = [], [], [], [], []
+    at = 0
+    for length, slot in zip(lengths, slot_of):
+        first.append(at)
+        count.append(length)
+        for a in range(0, length, size):
+            c_first.append(at + a)
+            c_count.append(min(size, length - a))
+        slots += [slot] * length
+        at += length
+    out = torch.full((n, heads * values), float("nan"), device="cuda")
+    scratch = torch.full((k.delta_chunk_floats(len(c_first), heads, keys, values),), float("nan"), device="cuda")
+    k.delta_rule_chunked(q, kk, v, decay, beta, out, live, stage, 0, ints(first), ints(count), len(first), ints(slots), ints(c_first),
+                         ints(c_count), len(c_first), scratch, heads, keys, values, heads_per_group=per_group, q_scale=0.25,
+                         unit_eps=1e-6)
+    q64, k64, v64, d64, b64 = (back(t) for t in (q, kk, v, decay, beta))
+    at = 0
+    for length, slot in zip(lengths, slot_of):
+        rows = slice(at, at + length)
+        for h in range(heads):
+            g = h // per_group
+            qh, kh = q64[rows, g * keys:(g + 1) * keys], k64[rows, g * keys:(g + 1) * keys]
+            qh = qh / np.sqrt((qh * qh).sum(axis=1, keepdims=True) + 1e-6) * 0.25
+            kh = kh / np.sqrt((kh * kh).sum(axis=1, keepdims=True) + 1e-6)
+            S = back(live[slot])[h * keys * values:(h + 1) * keys * values].reshape(keys, values).copy()
+            o = np.zeros((length, values))
+            for t in range(length):
+                S = np.exp(d64[at + t, h * keys:(h + 1) * keys])[:, None] * S
+                u = P.sigmoid(b64[at + t, h]) * (v64[at + t, h * values:(h + 1) * values] - S.T @ kh[t])
+                S = S + np.outer(kh[t], u)
+                o[t] = S.T @ qh[t]
+            scale = max(np.abs(o).max(), 1e-3)
+            np.testing.assert_allclose(back(out[rows, h * values:(h + 1) * values]), o, atol=5e-5 * scale, rtol=5e-5)
+            got = back(stage[slot])[h * keys * values:(h + 1) * keys * values].reshape(keys, values)
+            np.testing.assert_allclose(got, S, atol=5e-5 * max(np.abs(S).max(), 1e-3), rtol=5e-5)
+        at += length
+    assert torch.equal(stage[1], torch.zeros_like(stage[1]))
+
+
 def test_delta_rule_writes_before_it_reads_and_takes_back_what_a_key_held():
     """Inputs made so that a fault shows: one key written with value a and, much later and after many other orthogonal
     keys, written again with value b at full strength; a query for that key then reads b alone, and the token that
