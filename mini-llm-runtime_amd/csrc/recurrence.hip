@@ -378,12 +378,11 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(DeltaArgs a) {
 // and beta alone.  The first kernel (one workgroup per chunk and head, all side by side) leaves in scratch memory
 //     W = T (beta Khat) [DC, N],  Y = T (beta V) [DC, V],  B[t, s] = sum_i q_t[i] k_s[i] e^{c_t[i] - c_s[i]} (s <= t),
 //     Qhat[t] = q_t e^{c_t},  Kbar[s] = k_s e^{c_last - c_s},  G = e^{c_last};
-// the second (one workgroup per request, head and DELTA_CHUNK_COLS value channels) walks a request's chunks in
+// the second (one workgroup per request, head and 16 or 32 value channels) walks a request's chunks in
 // their order with the state in LDS:  U = Y - W S0;  O = Qhat S0 + B U;  S <- diag(G) S0 + Kbar^T U.
 // Every exponent is a difference c_t - c_s with s <= t or c_t itself, so nothing overflows however strong a decay
 // is.  The result differs from the token-by-token kernel's by 32-bit rounding.
 #define DELTA_CHUNK 32
-#define DELTA_CHUNK_COLS 32
 
 struct DeltaChunkArgs {
     DeltaArgs d;
@@ -503,83 +502,133 @@ __global__ __launch_bounds__(256) void delta_chunk_prepare_kernel(DeltaChunkArgs
     }
 }
 
+template <int VEC> struct alignas(4 * VEC) DeltaVec { float v[VEC]; };
+
+// VEC value channels a thread, 8 * VEC a workgroup: the narrower form fills the GPU when heads and value channels are few.
+template <int VEC>
 __global__ __launch_bounds__(256) void delta_chunk_scan_kernel(DeltaChunkArgs g) {
-    constexpr int C = DELTA_CHUNK, CS = DELTA_CHUNK + 1, COLS = DELTA_CHUNK_COLS;
+    constexpr int C = DELTA_CHUNK, CS = DELTA_CHUNK + 1, COLS = 8 * VEC;
+    constexpr int PER = DELTA_CHUNK * 128 / 256;           // elements of a [C][N] tile a thread moves, N <= 128
+    constexpr int PER_B = DELTA_CHUNK * DELTA_CHUNK / 256;
+    typedef DeltaVec<VEC> vec_t;
     const DeltaArgs& a = g.d;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     const int N = a.N, V = a.V, NS = N + 1;
     float* S_l = lds;                    // [N][COLS]
     float* U_l = S_l + N * COLS;         // [C][COLS]
-    float* buf = U_l + C * COLS;         // [C][NS]: W, then Qhat, then Kbar
-    float* B_l = buf + C * NS;           // [C][CS]
+    float* W_l = U_l + C * COLS;         // [C][NS]: W, then Kbar
+    float* Q_l = W_l + C * NS;           // [C][NS]: Qhat
+    float* B_l = Q_l + C * NS;           // [C][CS]
     float* G_l = B_l + C * CS;           // [N]
     const int seg = blockIdx.x, head = blockIdx.y, col0 = blockIdx.z * COLS;
     const int r0 = a.seg_first[seg], n = a.seg_count[seg];
     const int slot = a.slots[r0];
-    const int tid = threadIdx.x, t = tid >> 3, jq = (tid & 7) * 4;
+    const int tid = threadIdx.x, t = tid >> 3, jq = (tid & 7) * VEC;
     int chunk0 = 0;
     for (int s = 0; s < seg; ++s) chunk0 += (a.seg_count[s] + C - 1) / C;
     const size_t per = delta_chunk_floats(N, V);
     const size_t state_at = (size_t)slot * a.state_stride + (size_t)head * N * V;
+    const int tile = C * N;
+    int at_lds[PER];                                        // where this thread's tile elements go in LDS
+#pragma unroll
+    for (int r = 0; r < PER; ++r) {
+        const int idx = tid + 256 * r;
+        at_lds[r] = (idx / N) * NS + idx % N;
+    }
     for (int idx = tid; idx < N * COLS; idx += 256) {
         const int i = idx / COLS, c = col0 + idx % COLS;
         S_l[idx] = c < V ? a.live[state_at + (size_t)i * V + c] : 0.f;
     }
-    for (int c0 = 0, chunk = chunk0; c0 < n; c0 += C, ++chunk) {
-        const int nt = min(C, n - c0);
-        const float* base = g.scratch + ((size_t)chunk * a.heads + head) * per;
-        const float* W = base;
-        const float* Qh = W + (size_t)C * N;
-        const float* Kb = Qh + (size_t)C * N;
-        const float* Y = Kb + (size_t)C * N;
-        const float* B = Y + (size_t)C * V;
-        const float* G = B + C * C;
-        __syncthreads();                                    // the state is whole, the chunk before has been read
-        for (int idx = tid; idx < C * N; idx += 256) buf[(idx / N) * NS + idx % N] = W[idx];
-        for (int idx = tid; idx < C * C; idx += 256) B_l[(idx / C) * CS + idx % C] = B[idx];
-        for (int i = tid; i < N; i += 256) G_l[i] = G[i];
-        __syncthreads();
-        float u[4], o[4];
+    // a chunk's W, Qhat, B, G and Y are on their way into registers while the chunk before is worked on; Kbar while
+    // the chunk's own first products run
+    float w_next[PER], q_next[PER], k_next[PER], b_next[PER_B], y_next[VEC], g_next;
+    const float* base = g.scratch + ((size_t)chunk0 * a.heads + head) * per;
+    auto fetch = [&](const float* from) {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) u[e] = col0 + jq + e < V ? Y[(size_t)t * V + col0 + jq + e] : 0.f;
-        for (int i = 0; i < N; ++i) {
-            const float w = buf[t * NS + i];
-            const float4 s4 = *reinterpret_cast<const float4*>(S_l + i * COLS + jq);
-            u[0] -= w * s4.x; u[1] -= w * s4.y; u[2] -= w * s4.z; u[3] -= w * s4.w;
+        for (int r = 0; r < PER; ++r) {
+            const int idx = tid + 256 * r;
+            w_next[r] = idx < tile ? from[idx] : 0.f;
+            q_next[r] = idx < tile ? from[tile + idx] : 0.f;
         }
-        *reinterpret_cast<float4*>(U_l + t * COLS + jq) = make_float4(u[0], u[1], u[2], u[3]);
+        const float* Y = from + 3 * (size_t)tile;
+        const float* B = Y + (size_t)C * V;
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) y_next[e] = col0 + jq + e < V ? Y[(size_t)t * V + col0 + jq + e] : 0.f;
+#pragma unroll
+        for (int r = 0; r < PER_B; ++r) b_next[r] = B[tid + 256 * r];
+        g_next = tid < N ? B[C * C + tid] : 0.f;
+    };
+    fetch(base);
+    for (int c0 = 0; c0 < n; c0 += C) {
+        const int nt = min(C, n - c0);
+        const float* Kb = base + 2 * (size_t)tile;
+        __syncthreads();                                    // the state is whole, the tiles of the chunk before are read
+#pragma unroll
+        for (int r = 0; r < PER; ++r)
+            if (tid + 256 * r < tile) { W_l[at_lds[r]] = w_next[r]; Q_l[at_lds[r]] = q_next[r]; }
+#pragma unroll
+        for (int r = 0; r < PER_B; ++r) B_l[((tid + 256 * r) / C) * CS + (tid + 256 * r) % C] = b_next[r];
+        if (tid < N) G_l[tid] = g_next;
+        float u[VEC], o[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) { u[e] = y_next[e]; o[e] = 0.f; }
+#pragma unroll
+        for (int r = 0; r < PER; ++r) k_next[r] = tid + 256 * r < tile ? Kb[tid + 256 * r] : 0.f;
         __syncthreads();
-        for (int idx = tid; idx < C * N; idx += 256) buf[(idx / N) * NS + idx % N] = Qh[idx];
-        __syncthreads();
-        o[0] = o[1] = o[2] = o[3] = 0.f;
-        for (int i = 0; i < N; ++i) {
-            const float w = buf[t * NS + i];
-            const float4 s4 = *reinterpret_cast<const float4*>(S_l + i * COLS + jq);
-            o[0] += w * s4.x; o[1] += w * s4.y; o[2] += w * s4.z; o[3] += w * s4.w;
+        {
+            const float* wt = W_l + t * NS;
+            const float* qt = Q_l + t * NS;
+#pragma unroll 8
+            for (int i = 0; i < N; ++i) {
+                const float w = wt[i], qv = qt[i];
+                const vec_t s4 = *reinterpret_cast<const vec_t*>(S_l + i * COLS + jq);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) { u[e] -= w * s4.v[e]; o[e] += qv * s4.v[e]; }
+            }
         }
-        for (int s = 0; s <= t; ++s) {
-            const float w = B_l[t * CS + s];
-            const float4 u4 = *reinterpret_cast<const float4*>(U_l + s * COLS + jq);
-            o[0] += w * u4.x; o[1] += w * u4.y; o[2] += w * u4.z; o[3] += w * u4.w;
+        {
+            vec_t u4;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) u4.v[e] = u[e];
+            *reinterpret_cast<vec_t*>(U_l + t * COLS + jq) = u4;
+        }
+        __syncthreads();                                    // U is whole; W's tile has been read
+#pragma unroll
+        for (int r = 0; r < PER; ++r)
+            if (tid + 256 * r < tile) W_l[at_lds[r]] = k_next[r];
+        if (c0 + C < n) {
+            base += (size_t)a.heads * per;
+            fetch(base);
+        }
+        {
+            const float* bt = B_l + t * CS;
+#pragma unroll 4
+            for (int s = 0; s <= t; ++s) {
+                const float w = bt[s];
+                const vec_t u4 = *reinterpret_cast<const vec_t*>(U_l + s * COLS + jq);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) o[e] += w * u4.v[e];
+            }
         }
         if (t < nt) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
+            for (int e = 0; e < VEC; ++e)
                 if (col0 + jq + e < V) a.out[(size_t)(r0 + c0 + t) * ((size_t)a.heads * V) + head * V + col0 + jq + e] = o[e];
         }
-        __syncthreads();
-        for (int idx = tid; idx < C * N; idx += 256) buf[(idx / N) * NS + idx % N] = Kb[idx];
-        __syncthreads();
+        __syncthreads();                                    // Kbar is in W's place
         for (int i = t; i < N; i += C) {                   // (a thread's own elements of S: no other thread reads them now)
-            float4 s4 = *reinterpret_cast<const float4*>(S_l + i * COLS + jq);
+            vec_t s4 = *reinterpret_cast<const vec_t*>(S_l + i * COLS + jq);
             const float gi = G_l[i];
-            s4.x *= gi; s4.y *= gi; s4.z *= gi; s4.w *= gi;
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) s4.v[e] *= gi;
+#pragma unroll 8
             for (int s = 0; s < C; ++s) {
-                const float w = buf[s * NS + i];
-                const float4 u4 = *reinterpret_cast<const float4*>(U_l + s * COLS + jq);
-                s4.x += w * u4.x; s4.y += w * u4.y; s4.z += w * u4.z; s4.w += w * u4.w;
+                const float w = W_l[s * NS + i];
+                const vec_t u4 = *reinterpret_cast<const vec_t*>(U_l + s * COLS + jq);
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) s4.v[e] += w * u4.v[e];
             }
-            *reinterpret_cast<float4*>(S_l + i * COLS + jq) = s4;
+            *reinterpret_cast<vec_t*>(S_l + i * COLS + jq) = s4;
         }
     }
     __syncthreads();
@@ -737,9 +786,13 @@ int mlr_delta_rule_chunked(const void* q, long q_stride, const void* k, long k_s
     delta_chunk_prepare_kernel<<<dim3(chunks, heads), 256, lds1, stream>>>(g);
     int err = (int)hipGetLastError();
     if (err != 0) return err;
-    const size_t lds2 = sizeof(float) * ((size_t)n_keys * DELTA_CHUNK_COLS + (size_t)C * DELTA_CHUNK_COLS + (size_t)C * NS +
-                                         (size_t)C * (C + 1) + n_keys);
-    delta_chunk_scan_kernel<<<dim3(segments, heads, (n_values + DELTA_CHUNK_COLS - 1) / DELTA_CHUNK_COLS), 256, lds2, stream>>>(g);
+    // 32 value channels a workgroup where that fills the GPU, else 16
+    const bool wide = (long)segments * heads * ((n_values + 31) / 32) >= 256;
+    const int cols = wide ? 32 : 16;
+    const size_t lds2 = sizeof(float) * ((size_t)n_keys * cols + (size_t)C * cols + (size_t)2 * C * NS + (size_t)C * (C + 1) + n_keys);
+    const dim3 grid(segments, heads, (n_values + cols - 1) / cols);
+    if (wide) delta_chunk_scan_kernel<4><<<grid, 256, lds2, stream>>>(g);
+    else delta_chunk_scan_kernel<2><<<grid, 256, lds2, stream>>>(g);
     return (int)hipGetLastError();
 }
 

@@ -270,11 +270,11 @@ def test_delta_rule_carries_its_state_across_steps(dtype_name, heads, per_group,
 
 @pytest.mark.parametrize("dtype_name", DTYPES)
 @pytest.mark.parametrize("heads,per_group,keys,values", [(2, 1, 24, 40), (4, 2, 16, 24), (1, 1, 1, 1), (1, 1, 70, 65), (2, 2, 128, 100),
-                                                         (2, 1, 33, 64), (4, 1, 64, 32)])
+                                                         (2, 1, 33, 64), (4, 1, 64, 32), (48, 8, 8, 72)])
 def test_delta_rule_in_chunks_of_tokens(dtype_name, heads, per_group, keys, values):
     """Three requests of 150, 1 and 37 tokens in one step, from states that are not zero, cut into chunks of the
     kernel's size; decays from none at all to e^-30 a token (no quotient of decays may be formed); outputs and staged
-    states against the plain rule continued from the same states."""
+    states against the plain rule continued from the same states.  (Many heads: the kernel's wider workgroups.)"""
     from mini_llm_runtime_amd.kernels import Kernels
     dtype = DTYPES[dtype_name]
     k = Kernels(dtype)
