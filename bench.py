@@ -602,7 +602,7 @@ class TigelornBench(Bench):
         layers = [turn[i % 4] for i in range(self.layers)]
         kinds = [layer["type"] for layer in layers]
         self.cfg = config_from_dict(dict(architecture="Tigelorn", vocab=d["vocab"], width=d["width"], norm=dict(eps=1e-5),
-                                         embedding=dict(bigram=dict(buckets=16381, mul_prev=1000003, mul_cur=31)), layers=layers))
+                                         embedding=dict(bigram=dict(buckets=16381, mul_prev=1000003, mul_cur=29)), layers=layers))
         self.model = DecoderModel(self.cfg, random_tensors_on_device(expected_tensors(self.cfg), 0, self.dtype, "cuda"),
                                   self.dtype, "cuda:0")
         self.weights_from = "drawn on the GPU"

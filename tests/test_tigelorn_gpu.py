@@ -75,7 +75,7 @@ CONFIGS = {
                               dense(latent(8, 32, 16, 32, 64, 48), 160),
                               dense(delta(4, 4, 64, 32, 4), None),
                               dense(parallel(window(4, 4, 32, 16, 1000, 32, base=1e6), decayed(16, 64, [0.9, 0.97])), None),
-                              dense(latent(8, 32, 16, 32, 64, 48), 160, weights_of=1)], pairs=(251, 123456789, 7)),
+                              dense(latent(8, 32, 16, 32, 64, 48), 160, weights_of=1)], pairs=(251, 123456789, 9)),
     "state_only": model(64, 48, [dense(delta(2, 1, 24, 16, 3), 64), dense(delta(2, 2, 8, 8, 2), None)]),
 }
 LENGTHS = [70, 33, 150, 17, 64, 129, 2, 45]
@@ -548,7 +548,7 @@ def plain_attend(q, keys, values, positions, size, scale, group):
 
 
 @pytest.mark.parametrize("dtype_name", DTYPES)
-@pytest.mark.parametrize("size", [37, 1, 64, 136, None])
+@pytest.mark.parametrize("size", [37, 1, 64, 150, None])
 @pytest.mark.parametrize("heads,kv,dim,vdim,shared,page", [(4, 2, 32, 16, False, 8), (3, 1, 20, 70, False, 4), (6, 1, 48, 32, True, 16)])
 def test_softmax_attention_finds_one_key_wherever_it_lies(dtype_name, size, heads, kv, dim, vdim, shared, page):
     """One key among 300 is made to stand out for one query: the query's output is that key's value when the window

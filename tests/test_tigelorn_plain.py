@@ -296,7 +296,7 @@ def test_configuration_refuses_what_it_cannot_mean():
 def test_position_part_computes_the_plain_frequencies_in_32_bit():
     from mini_llm_runtime_amd.config.specs import FrequencyStretch, PositionSpec
     from mini_llm_runtime_amd.parts.rope import Rope
-    for dims, base, scaling in ((32, 10000.0, dict(factor=4.0, original=2048, fast=32.0, slow=1.0)), (6, 50.0, None),
+    for dims, base, scaling in ((24, 5000.0, dict(factor=3.0, original=1024, fast=16.0, slow=1.0)), (6, 50.0, None),
                                 (16, 100.0, dict(factor=1.5, original=64, fast=8.0, slow=2.0))):
         stretch = FrequencyStretch(**scaling) if scaling else None
         freq, amp = Rope(PositionSpec("rope", dims, base, interleaved=True, stretch=stretch)).frequencies()
