@@ -210,7 +210,7 @@ struct SkinnyEpilogue {
     int cols;                 // PAIR: the output columns of a workgroup, 17..32 (otherwise 16, whatever this says)
     int ss_stride;            // floats between the rows of ss_out (its capacity: a strip of 16 a part)
     float glu_limit;          // GATED: > 0: the clamped gate g = min(gate, limit), u = clamp(up, +-limit),
-    float glu_slope;          //        y = g sigmoid(slope g) (u + 1); 0: y = silu(gate) up
+    float glu_slope;          //        y = g sigmoid(slope g) (u + 1); 0: y = silu(gate) up; < 0: y = gelu_tanh(gate) up
 };
 
 // PAIR: a workgroup owns `cols` (17..32) output columns, two strips side by side, the second one partly
@@ -442,6 +442,9 @@ __global__ __launch_bounds__(SKINNY_WAVES * 64) void gemm_skinny_kernel(const __
                     const float gg = fminf(v[0], epi.glu_limit);
                     const float uu = fminf(fmaxf(v[NW - 1], -epi.glu_limit), epi.glu_limit);
                     y = (gg / (1.0f + expf(-epi.glu_slope * gg))) * (uu + 1.0f);
+                } else if (epi.glu_limit < 0.f) {
+                    const float gg = v[0];
+                    y = 0.5f * gg * (1.0f + tanhf(0.7978845608028654f * (gg + 0.044715f * gg * gg * gg))) * v[NW - 1];
                 } else {
                     y = (v[0] / (1.0f + expf(-v[0]))) * v[NW - 1];
                 }
@@ -991,6 +994,19 @@ extern "C" int mlr_gemm_gated_clamped(const void* a, const void* w, void* out, i
     SkinnyEpilogue epi{};
     epi.glu_limit = limit;
     epi.glu_slope = slope;
+    if (M <= 16) return launch_skinny<1, true>(a, w, out, M, N, K, 0, stream, epi);
+    if (M <= 32) return launch_skinny<2, true>(a, w, out, M, N, K, 0, stream, epi);
+    if (M <= 64) return launch_skinny<4, true>(a, w, out, M, N, K, 0, stream, epi);
+    return 1;
+}
+
+// out[M, N] = gelu_tanh(a . w[0:N]^T) * (a . w[N:2N]^T), gelu_tanh(g) = 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3))):
+// the gate as the epilogue of the weight-streaming kernels, up to 64 rows.  Returns 1 for more rows.
+extern "C" int mlr_gemm_gated_gelu_tanh(const void* a, const void* w, void* out, int M, int N, int K, hipStream_t stream) {
+    if (M <= 0 || N <= 0) return 0;
+    if (K <= 0) return -1;
+    SkinnyEpilogue epi{};
+    epi.glu_limit = -1.0f;
     if (M <= 16) return launch_skinny<1, true>(a, w, out, M, N, K, 0, stream, epi);
     if (M <= 32) return launch_skinny<2, true>(a, w, out, M, N, K, 0, stream, epi);
     if (M <= 64) return launch_skinny<4, true>(a, w, out, M, N, K, 0, stream, epi);

@@ -379,6 +379,20 @@ class Kernels:
         _ok(fn(_p(a), _p(w), _p(out), _c_int(m), _c_int(two_n // 2), _c_int(k), _c_float(limit), _c_float(slope), _stream()),
             "gemm_gated_clamped")
 
+    @timed("gemm", _gemm_work)
+    def gemm_gated_gelu_tanh(self, a, w, out):
+        """out[M, N] = gelu_tanh(a . w[:N]^T) * (a . w[N:]^T), w = [gate; up] stacked: the tanh form of gelu fused into
+        the weight-streaming projection, up to 64 rows (bfloat16)."""
+        _need(self.dtype == torch.bfloat16 and a.shape[0] <= 64, "gemm_gated_gelu_tanh: bfloat16, up to 64 rows")
+        _tensor(a, "a", self.dtype, ndim=2)
+        _tensor(w, "w", self.dtype, ndim=2)
+        m, k = a.shape
+        two_n, k2 = w.shape
+        _need(k == k2 and two_n % 2 == 0, "gemm_gated_gelu_tanh: sizes do not fit")
+        _tensor(out, "out", self.dtype, (m, two_n // 2))
+        _ok(self._lib("gemm").mlr_gemm_gated_gelu_tanh(_p(a), _p(w), _p(out), _c_int(m), _c_int(two_n // 2), _c_int(k),
+                                                       _stream()), "gemm_gated_gelu_tanh")
+
     # -- an RMSNorm handed from one projection to the next (few rows) ------------------------------
     HANDOFF_MAX_ROWS = 16
 

@@ -1,6 +1,7 @@
 """SwiGLU feed-forward: out = (silu(x Wgate^T) * (x Wup^T)) Wdown^T with silu(g) = g / (1 + exp(-g))
 (src/minillm/runtime.cpp:323-336).  Gate and up are one stacked projection.  The gate's activation is the spec's:
-silu, or gelu_tanh (0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))), which takes the unfused path."""
+silu, or gelu_tanh (0.5 g (1 + tanh(sqrt(2/pi) (g + 0.044715 g^3)))); for few rows either rides on the projection,
+the norm handed between projections is silu's alone."""
 from __future__ import annotations
 
 import torch
@@ -61,6 +62,8 @@ class SwiGluMlp:
         act = ctx.workspace.get("act", (m, s.intermediate), x.dtype)
         if s.activation == "silu" and ctx.kernels.gated_silu_fused(m, s.hidden):
             ctx.kernels.gemm_gated_silu(x, self.gate_up, act)      # few rows: the activation rides on the projection
+        elif s.activation == "gelu_tanh" and m <= 64 and ctx.kernels.streams_weight(m, s.hidden):
+            ctx.kernels.gemm_gated_gelu_tanh(x, self.gate_up, act)
         else:
             gate_up = ctx.workspace.get("gate_up", (m, 2 * s.intermediate), x.dtype)
             ctx.kernels.gemm(x, self.gate_up, gate_up)
