@@ -37,7 +37,8 @@ DELTA_UNIT_EPS = 1e-6          # inside the root that makes q and k of the delta
 
 def _rotation(m, where, interleaved, dims=None):
     rot = _object(m, "rot", where)
-    n = _int(rot, "dims", where + "rot.")
+    # (where the mixer fixes how many channels turn, `dims` may be left out)
+    n = dims if dims is not None and rot.get("dims") is None else _int(rot, "dims", where + "rot.")
     if n % 2 != 0 or (dims is not None and n != dims):
         raise ConfigError(f"config.json: {where}rot.dims {n} must be even" + (f" and equal rot_dim {dims}" if dims else ""))
     stretch = None
