@@ -14,7 +14,7 @@ from typing import Optional, Tuple
 
 @dataclass(frozen=True)
 class NormSpec:
-    kind: str                 # key in the norm registry, e.g. "rmsnorm"
+    kind: str                 # key in the norm registry, e.g. "rmsnorm"; "tanh_norm" takes no statistics and no eps
     size: int
     eps: float
     weight_offset: float = 0.0    # the factor is weight_offset + the stored weight (1: a weight stored around zero)
@@ -88,6 +88,8 @@ class DiffAttentionSpec:
     softcap: Optional[float] = None           # score <- softcap * tanh(score / softcap)
     q_temperature: Optional[QueryTemperature] = None
     gate: Optional[str] = "sigmoid"           # activation of the output gate (None: no gate)
+    position: Optional[PositionSpec] = None   # turns the first `dim` channels of every map of q and k
+    mask: Optional["MaskSpec"] = None         # None: every earlier key
 
 
 @dataclass(frozen=True)
@@ -179,6 +181,7 @@ class LatentAttentionSpec:
     mask: Optional[MaskSpec] = None
     sink: bool = True
     q_rank: Optional[int] = None                 # queries through a normed latent of their own: Wuq norm(Wdq x)
+    head_gate: Optional[str] = None              # "sigmoid": a head's output times sigmoid(Wg x)[head], Wg [heads, hidden]
 
 
 @dataclass(frozen=True)
@@ -215,6 +218,8 @@ class DeltaRuleSpec:
     unit_eps: float = 1e-6
     decay_rank: Optional[int] = None      # None: the file's tensors say
     gate_rank: Optional[int] = None
+    decay: str = "channel_low_rank"       # "head": one decay a head, g = exp(-exp(A_log) softplus(Wa x + dt_bias)), Wa [heads, hidden]
+    gate: str = "low_rank_sigmoid"        # "silu": the read-out times silu(Wg x), Wg a full matrix
 
 
 @dataclass(frozen=True)
@@ -251,6 +256,9 @@ class RoutedMlpSpec:
     activation: str = "relu_squared"
     score: str = "sigmoid"
     renormalize: bool = False
+    gated: bool = False           # an expert is down(act(gate x) * (up x)) with tensors e<i>.gate beside e<i>.up
+    correction: bool = False      # the choice goes by s + a stored number an expert (`correction`), the weights by s
+    route_scale: float = 1.0      # factor on the chosen weights
 
 
 @dataclass(frozen=True)
@@ -260,6 +268,8 @@ class LayerSpec:
     mixer: object             # any mixer spec with a `kind`
     norm2: Optional[NormSpec]     # None with `ffn` None: a layer without a feed-forward
     ffn: object               # any feed-forward spec with a `kind`
+    norm1_after: Optional[NormSpec] = None    # block "sandwich": the norm of what the mixer gives, before the residual sum
+    norm2_after: Optional[NormSpec] = None    # likewise behind the feed-forward
 
 
 @dataclass(frozen=True)
@@ -269,6 +279,8 @@ class LayerRun:
     layer: int
     cache: int
     write_cache: bool = True
+    add_embedding: bool = False   # the embedding's output (the stream as it was before the first run) is added to
+                                  # the stream right before this run: the start of a further pass over looped layers
 
 
 @dataclass(frozen=True)
@@ -297,6 +309,7 @@ class HeadSpec:
     hidden: int
     tied: bool = False        # no tensor of its own: the embedding's table
     scale: float = 1.0        # factor on the logits (kind "scaled_head")
+    softcap: Optional[float] = None   # logits <- softcap * tanh(logits / softcap) (kind "capped_head")
 
 
 @dataclass(frozen=True)

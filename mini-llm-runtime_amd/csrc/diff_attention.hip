@@ -5,7 +5,10 @@
 // is o = a1 - lam * a2, divided by its root mean square over the value channels (eps inside the root), times
 // out_scale, times an activation of the head's gate.  Scores: (q . k) * scale * temp(p), the query's factor
 // temp(p) = 1 + coef * ln(floor((p + 1) / every) + 1) growing with its position p; then, with a cap,
-// score <- cap * tanh(score / cap); position p sees the keys 0 .. p.  All of this is 32-bit.
+// score <- cap * tanh(score / cap); position p sees the keys 0 .. p, or with a mask rule only the last `mask_size`
+// of them (window) or those of its own block of `mask_size` positions counted from 0 (chunk).  All of this is
+// 32-bit.  Queries and keys may be rotated on their way (`diff_qkv_prep_kernel`): the first `rot` channels of each
+// map of each head, in pairs (j, j + rot / 2) or (2 j, 2 j + 1), by the angles of the position's table row.
 //
 // Cache of one layer: keys pages[num_pages][kv_heads][page_size][2 * head_dim]; values transposed within a
 // page, pages[num_pages][kv_heads][value_dim][page_size], so that the keys of one channel lie side by side (the
@@ -43,7 +46,18 @@ struct DiffArgs {
     // which rows: null: blockIdx.x is the batch row; else blockIdx.x = group * group_tokens + i stands for row
     // group_first[group] + i while i < group_count[group] (partial results are indexed by blockIdx.x)
     const int32_t* group_first; const int32_t* group_count; int group_tokens;
+    int mask_kind, mask_size;                  // 0: every earlier key; 1: the last mask_size positions; 2: the query's block
 };
+
+#define MASK_NONE 0
+#define MASK_WINDOW 1
+#define MASK_CHUNK 2
+// The first key that a query at `pos` sees (never decreasing in pos).
+__device__ __forceinline__ int first_key(const DiffArgs& a, int pos) {
+    if (a.mask_kind == MASK_WINDOW) return max(0, pos - a.mask_size + 1);
+    if (a.mask_kind == MASK_CHUNK) return (pos / a.mask_size) * a.mask_size;
+    return 0;
+}
 
 __device__ __forceinline__ int diff_row(const DiffArgs& a) {
     if (a.group_first == nullptr) return blockIdx.x;
@@ -72,6 +86,55 @@ __global__ void diff_kv_write_kernel(const elem_t* __restrict__ k, long k_stride
     }
 }
 
+// The rotation of a step's queries and keys and the write of its keys and values: a workgroup a token.  q is turned
+// in place (columns of the projection's output); keys are turned on their way into the pages.  `rope` [positions,
+// rot]: cosines in the first half of a row, sines in the second; every map of every head turns its first `rot`
+// channels (rot <= head_dim, even), the others pass.  32-bit inside; rope null: nothing turns.
+__global__ void diff_qkv_prep_kernel(elem_t* __restrict__ q, long q_stride, const elem_t* __restrict__ k, long k_stride,
+                                     const elem_t* __restrict__ v, long v_stride, elem_t* __restrict__ k_pages,
+                                     elem_t* __restrict__ v_pages, const int32_t* __restrict__ block_table, int max_blocks,
+                                     const int32_t* __restrict__ slots, const int32_t* __restrict__ positions,
+                                     const float* __restrict__ rope, int rot, int interleaved, int q_heads, int kv_heads,
+                                     int head_dim, int value_dim, int page_size, int write_cache) {
+    const int m = blockIdx.x;
+    const int pos = positions[m];
+    const int block = pos / page_size, at = pos % page_size;
+    const int page = (write_cache && block < max_blocks) ? block_table[(size_t)slots[m] * max_blocks + block] : -1;
+    const int half = rot / 2;
+    const float* angle = rope != nullptr ? rope + (size_t)pos * rot : nullptr;
+    // pairs of the queries: (head, map) x rot / 2
+    if (angle != nullptr) {
+        elem_t* qr = q + (size_t)m * q_stride;
+        for (int i = threadIdx.x; i < q_heads * 2 * half; i += blockDim.x) {
+            const int hm = i / half, j = i % half;
+            const int d0 = interleaved ? 2 * j : j, d1 = interleaved ? 2 * j + 1 : j + half;
+            elem_t* base = qr + (size_t)hm * head_dim;
+            const float x = to_float(base[d0]), y = to_float(base[d1]), c = angle[j], s = angle[half + j];
+            base[d0] = from_float<elem_t>(turn_x(x, y, c, s));
+            base[d1] = from_float<elem_t>(turn_y(x, y, c, s));
+        }
+    }
+    if (page < 0) return;                      // (no page: nothing is written)
+    const int key_dim = 2 * head_dim;
+    for (int i = threadIdx.x; i < kv_heads * key_dim; i += blockDim.x) {
+        const int g = i / key_dim, d = i % key_dim, dm = d % head_dim;
+        const elem_t* src = k + (size_t)m * k_stride;
+        float val = to_float(src[i]);
+        if (angle != nullptr && dm < rot) {
+            const int j = interleaved ? dm / 2 : dm % half;
+            const bool second = interleaved ? (dm & 1) : dm >= half;
+            const int other = interleaved ? (second ? i - 1 : i + 1) : (second ? i - half : i + half);
+            const float o = to_float(src[other]), c = angle[j], s = angle[half + j];
+            val = second ? turn_y(o, val, c, s) : turn_x(val, o, c, s);
+        }
+        k_pages[(((size_t)page * kv_heads + g) * page_size + at) * key_dim + d] = from_float<elem_t>(val);
+    }
+    for (int i = threadIdx.x; i < kv_heads * value_dim; i += blockDim.x) {
+        const int g = i / value_dim, d = i % value_dim;
+        v_pages[(((size_t)page * kv_heads + g) * value_dim + d) * page_size + at] = v[(size_t)m * v_stride + i];
+    }
+}
+
 __device__ __forceinline__ float query_temperature(int pos, float coef, float every) {
     return coef != 0.f ? 1.0f + coef * logf(floorf((float)(pos + 1) / every) + 1.0f) : 1.0f;
 }
@@ -89,9 +152,9 @@ __global__ __launch_bounds__(64) void diff_attention_partial_kernel(DiffArgs a) 
     const int D = a.head_dim, V = a.value_dim;
     const int kvh = head / (a.q_heads / a.kv_heads);
     const int pos = a.positions[m], slot = a.slots[m];
-    int kbegin = 0, kend = pos + 1;
+    int kbegin = first_key(a, pos), kend = pos + 1;
     if (a.max_splits > 1) {
-        kbegin = split * a.split_keys;
+        kbegin = max(kbegin, split * a.split_keys);
         kend = min(kend, (split + 1) * a.split_keys);
     }
     float* dst = a.partial + (((size_t)blockIdx.x * a.q_heads * 2 + hm) * a.max_splits + split) * (V + 2);
@@ -178,10 +241,12 @@ __global__ __launch_bounds__(64) void diff_attention_combine_kernel(DiffArgs a) 
     if (m < 0) return;
     const int V = a.value_dim;
     const int pos = a.positions[m];
-    const int n = a.max_splits > 1 ? min(a.max_splits - 1, pos / a.split_keys) + 1 : 1;
+    // the ranges that hold keys this token sees: from its first key's range to its own position's
+    const int s0 = a.max_splits > 1 ? min(a.max_splits - 1, first_key(a, pos) / a.split_keys) : 0;
+    const int n = (a.max_splits > 1 ? min(a.max_splits - 1, pos / a.split_keys) + 1 : 1) - s0;
     float maps[2][MAX_V_REGS];
     for (int map = 0; map < 2; ++map) {
-        const float* base = a.partial + ((size_t)blockIdx.x * a.q_heads * 2 + head * 2 + map) * a.max_splits * (V + 2);
+        const float* base = a.partial + (((size_t)blockIdx.x * a.q_heads * 2 + head * 2 + map) * a.max_splits + s0) * (V + 2);
         float gmax = -INFINITY;
         __syncthreads();
         for (int s = lane; s < n; s += 64) {
@@ -273,10 +338,15 @@ __device__ __forceinline__ void diff_tiles_group(const DiffArgs& a, const int32_
     const bool wave_active = tblock < token_blocks && head0 < g && tblock * tokens_per_wave < ntok;
     const bool col_valid = wave_active && col < tokens_per_wave * col_heads && hh < g && tok < ntok;
     const int pos = pos0 + tok;
-    const int kend_c = col_valid ? pos + 1 : 0;       // keys this column sees: [0, kend_c)
-    const int ke = pos0 + ntok;                       // keys the workgroup walks: [0, ke)
+    const int kend_c = col_valid ? pos + 1 : 0;       // keys this column sees: [kbeg_c, kend_c)
+    const int kbeg_c = first_key(a, pos);
+    const int ke = pos0 + ntok;                       // keys the workgroup walks: [first_key(pos0) in whole tiles, ke)
     const int wave_hi = wave_active ? pos0 + min(ntok, tblock * tokens_per_wave + tokens_per_wave) : 0;
     const int wave_first_kend = pos0 + tblock * tokens_per_wave + 1;
+    // (first_key never decreases with the position: the wavefront's first token sees the earliest keys of its
+    // columns, its last token's first key is seen by all of them)
+    const int wave_first_kbeg = first_key(a, pos0 + tblock * tokens_per_wave);
+    const int wave_last_kbeg = wave_active ? first_key(a, wave_hi - 1) : 0;
     const __bf16* q = reinterpret_cast<const __bf16*>(a.q);
     const __bf16* kp_base = reinterpret_cast<const __bf16*>(a.k_pages);
     const __bf16* vp_base = reinterpret_cast<const __bf16*>(a.v_pages);
@@ -311,11 +381,12 @@ __device__ __forceinline__ void diff_tiles_group(const DiffArgs& a, const int32_
     // with key ranges: this workgroup walks [split * split_keys, (split + 1) * split_keys) (multiples of 32) and
     // leaves partial results for the merge
     const int split = blockIdx.z;
-    const int k_lo = a.max_splits > 1 ? split * a.split_keys : 0;
+    const int group_lo = (first_key(a, pos0) / TKEYS) * TKEYS;      // (the group's first token sees the earliest keys)
+    const int k_lo = a.max_splits > 1 ? max(split * a.split_keys, group_lo) : group_lo;
     const int k_hi = a.max_splits > 1 ? min(ke, (split + 1) * a.split_keys) : ke;
     if (k_lo >= k_hi) return;                         // (a range beyond the group's keys: the merge does not read it)
     // page ids of the range first, so that a tile's loads do not wait for a load of the block table
-    const int first_page = k_lo / P;                  // (k_lo is a multiple of 64; pages of 8 k tokens)
+    const int first_page = k_lo / P;                  // (the page that holds key k_lo)
     {
         const int n_pages = min(TILES_PAGE_CACHE, (k_hi + P - 1) / P - first_page);
         for (int i = threadIdx.x; i < n_pages; i += 256) page_lds[i] = first_page + i < a.max_blocks ? table[first_page + i] : -1;
@@ -398,8 +469,8 @@ __device__ __forceinline__ void diff_tiles_group(const DiffArgs& a, const int32_
         }
     };
     auto compute = [&](int tb) {
-        if (!wave_active || tb >= wave_hi) return;
-        const bool interior = tb + TKEYS <= wave_first_kend;
+        if (!wave_active || tb >= wave_hi || tb + TKEYS <= wave_first_kbeg) return;
+        const bool interior = tb + TKEYS <= wave_first_kend && tb >= wave_last_kbeg;
 #pragma unroll
         for (int map = 0; map < 2; ++map) {
             if (map_split && map != my_map) continue;
@@ -426,7 +497,7 @@ __device__ __forceinline__ void diff_tiles_group(const DiffArgs& a, const int32_
                         x = cap2 - 2.0f * cap2 * __builtin_amdgcn_rcpf(e + 1.0f);
                     }
                     const int key = tb + 16 * j + 4 * b + r;
-                    sv[j][r] = (interior || key < kend_c) ? x : -INFINITY;
+                    sv[j][r] = (interior || (key < kend_c && key >= kbeg_c)) ? x : -INFINITY;
                 }
             float tile_max = fmaxf(fmaxf(fmaxf(sv[0][0], sv[0][1]), fmaxf(sv[0][2], sv[0][3])),
                                    fmaxf(fmaxf(sv[1][0], sv[1][1]), fmaxf(sv[1][2], sv[1][3])));
@@ -580,12 +651,26 @@ int mlr_diff_kv_write(const void* k, long k_stride, const void* v, long v_stride
     return (int)hipGetLastError();
 }
 
+int mlr_diff_qkv_prep(void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride, void* k_pages,
+                      void* v_pages, const int32_t* block_table, int max_blocks, const int32_t* slots,
+                      const int32_t* positions, const float* rope, int rot, int interleaved, int rows, int q_heads,
+                      int kv_heads, int head_dim, int value_dim, int page_size, int write_cache, hipStream_t stream) {
+    if (rows <= 0) return 0;
+    if (rope != nullptr && (rot < 2 || rot % 2 != 0 || rot > head_dim)) return -1;
+    diff_qkv_prep_kernel<<<rows, 256, 0, stream>>>((elem_t*)q, q_stride, (const elem_t*)k, k_stride, (const elem_t*)v, v_stride,
+                                                   (elem_t*)k_pages, (elem_t*)v_pages, block_table, max_blocks, slots,
+                                                   positions, rope, rot, interleaved, q_heads, kv_heads, head_dim, value_dim,
+                                                   page_size, write_cache);
+    return (int)hipGetLastError();
+}
+
 int mlr_diff_attention(const void* q, long q_stride, const void* k_pages, const void* v_pages, const int32_t* block_table,
                        int max_blocks, const int32_t* slots, const int32_t* positions, const void* gate, long gate_stride,
                        void* out, float* partial, int rows, int q_heads, int kv_heads, int head_dim, int value_dim,
                        int page_size, float scale, float softcap, float temp_coef, float temp_every, float lam,
                        float out_scale, float eps, int split_keys, int max_splits, const int32_t* group_first,
-                       const int32_t* group_count, int groups, int group_tokens, hipStream_t stream) {
+                       const int32_t* group_count, int groups, int group_tokens, int mask_kind, int mask_size,
+                       hipStream_t stream) {
     // (with groups: `rows` = groups * group_tokens places, of which those beyond a group's count stay idle)
     if (group_first != nullptr) rows = groups * group_tokens;
     if (rows <= 0) return 0;
@@ -593,10 +678,11 @@ int mlr_diff_attention(const void* q, long q_stride, const void* k_pages, const 
     if (max_splits < 1) max_splits = 1;
     if (max_splits > 1 && (split_keys <= 0 || split_keys % TILE_KEYS != 0 || max_splits > COMBINE_MAX_SPLITS)) return -2;
     if (temp_coef != 0.f && !(temp_every > 0.f)) return -3;
+    if (mask_kind < MASK_NONE || mask_kind > MASK_CHUNK || (mask_kind != MASK_NONE && mask_size < 1)) return -5;
     DiffArgs a{(const elem_t*)q, q_stride, (const elem_t*)k_pages, (const elem_t*)v_pages, block_table, slots, positions,
                (const elem_t*)gate, gate_stride, (elem_t*)out, partial, max_blocks, q_heads, kv_heads, head_dim, value_dim,
                page_size, split_keys, max_splits, scale, softcap, temp_coef, temp_every, lam, out_scale, eps,
-               group_first, group_count, group_tokens};
+               group_first, group_count, group_tokens, mask_kind, mask_size};
     diff_attention_partial_kernel<<<dim3(rows, q_heads * 2, max_splits), 64, 0, stream>>>(a);
     int err = (int)hipGetLastError();
     if (err != 0) return err;
@@ -616,9 +702,13 @@ int mlr_diff_attention_tiles(const void* q, long q_stride, const void* k_pages, 
                              const int32_t* group_ntok, int groups, int group_tokens, int q_heads, int kv_heads,
                              int head_dim, int value_dim, int page_size, float scale, float softcap, float temp_coef,
                              float temp_every, float lam, float out_scale, float eps, int split_keys, int max_splits,
-                             int max_context, hipStream_t stream) {
+                             int max_context, int mask_kind, int mask_size, hipStream_t stream) {
 #if MLR_BF16
     if (groups <= 0) return 0;
+    if (mask_kind < MASK_NONE || mask_kind > MASK_CHUNK || (mask_kind != MASK_NONE && mask_size < 1)) return -5;
+    // (behind a mask a workgroup walks the keys of its tokens' window or block only)
+    if (mask_kind != MASK_NONE && mask_size + group_tokens + 2 * TILE_KEYS < max_context)
+        max_context = mask_size + group_tokens + 2 * TILE_KEYS;
     // the keys one workgroup walks (a range, or without ranges the longest context of the step) lie in at most
     // TILES_PAGE_CACHE pages, whose ids it keeps in LDS
     if (((max_splits > 1 ? split_keys : max_context) + page_size - 1) / page_size + 1 > TILES_PAGE_CACHE) return -4;
@@ -641,7 +731,7 @@ int mlr_diff_attention_tiles(const void* q, long q_stride, const void* k_pages, 
     DiffArgs a{(const elem_t*)q, q_stride, (const elem_t*)k_pages, (const elem_t*)v_pages, block_table, slots, positions,
                (const elem_t*)gate, gate_stride, (elem_t*)out, partial, max_blocks, q_heads, kv_heads, head_dim, value_dim,
                page_size, split_keys, max_splits, scale, softcap, temp_coef, temp_every, lam, out_scale, eps,
-               group_row0, group_ntok, group_tokens};
+               group_row0, group_ntok, group_tokens, mask_kind, mask_size};
     const int nch = (head_dim + 31) / 32;
     int err;
     if (nch == 1) err = launch_tiles<1>(a, group_row0, group_ntok, groups, ch, wh, tbw, ms, stream);

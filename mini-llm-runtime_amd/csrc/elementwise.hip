@@ -717,6 +717,89 @@ __global__ void scale_float_kernel(float* __restrict__ x, float factor, size_t c
         x[i] *= factor;
 }
 
+// ---- a norm without statistics: y = tanh(alpha x) w + b, element by element, 32-bit ---------------------------
+__device__ __forceinline__ float tanh_norm(float x, float alpha, float w, float b) { return __builtin_fmaf(tanhf(alpha * x), w, b); }
+
+// x = h[row] + delta[row] (delta may be null; written back to h when write_h), out[r] = norm(x) for row = rows[r]
+// (rows null: r).  One thread takes VEC consecutive elements (width a multiple of VEC).
+template <int VEC>
+__global__ void tanh_norm_rows_kernel(float* __restrict__ h, const elem_t* __restrict__ delta, const float* __restrict__ w,
+                                      const float* __restrict__ b, float alpha, elem_t* __restrict__ out,
+                                      const int32_t* __restrict__ rows, size_t n_out, int width, int write_h) {
+    const size_t per_row = width / VEC, total = n_out * per_row;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / per_row, c = (i % per_row) * VEC;
+        const size_t row = rows != nullptr ? (size_t)rows[r] : r;
+        float x[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) x[e] = h[row * width + c + e];
+        if (delta != nullptr) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) x[e] += to_float(delta[row * width + c + e]);
+            if (write_h) {
+#pragma unroll
+                for (int e = 0; e < VEC; ++e) h[row * width + c + e] = x[e];
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) out[r * width + c + e] = from_float<elem_t>(tanh_norm(x[e], alpha, w[c + e], b[c + e]));
+    }
+}
+
+// h += norm_a(delta) (+ extra, a float matrix like h, when given); then, when out is given, out = norm_n(h): the norm
+// behind a sublayer, the residual sum and the norm in front of the next sublayer in one pass over the row.
+template <int VEC>
+__global__ void tanh_norm_add_kernel(const elem_t* __restrict__ delta, const float* __restrict__ wa, const float* __restrict__ ba,
+                                     float alpha_a, float* __restrict__ h, const float* __restrict__ extra,
+                                     const float* __restrict__ wn, const float* __restrict__ bn, float alpha_n,
+                                     elem_t* __restrict__ out, size_t n_rows, int width) {
+    const size_t per_row = width / VEC, total = n_rows * per_row;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t at = (i / per_row) * width + (i % per_row) * VEC;
+        const int c = (int)((i % per_row) * VEC);
+        float x[VEC];
+#pragma unroll
+        for (int e = 0; e < VEC; ++e) {
+            x[e] = h[at + e] + tanh_norm(to_float(delta[at + e]), alpha_a, wa[c + e], ba[c + e]);
+            if (extra != nullptr) x[e] += extra[at + e];
+            h[at + e] = x[e];
+        }
+        if (out != nullptr) {
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) out[at + e] = from_float<elem_t>(tanh_norm(x[e], alpha_n, wn[c + e], bn[c + e]));
+        }
+    }
+}
+
+// h += extra (float matrices of the same size).
+__global__ void residual_add_float_kernel(float* __restrict__ h, const float* __restrict__ extra, size_t count) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+        h[i] += extra[i];
+}
+
+// dst = src (float matrices of the same size): the copy of the residual stream that later passes add again.
+__global__ void copy_float_kernel(const float* __restrict__ src, float* __restrict__ dst, size_t count) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+        dst[i] = src[i];
+}
+
+// x <- cap * tanh(x / cap) (float values, logits for instance).
+__global__ void tanh_cap_kernel(float* __restrict__ x, float cap, size_t count) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += (size_t)gridDim.x * blockDim.x)
+        x[i] = cap * tanhf(x[i] / cap);
+}
+
+// out[m, head * part + c] = x[m, head * part + c] * sigmoid(gate[m * gate_stride + head]): one gate a head.
+__global__ void head_gate_mul_kernel(const elem_t* __restrict__ x, const elem_t* __restrict__ gate, long gate_stride,
+                                     elem_t* __restrict__ out, size_t rows, int width, int part) {
+    const size_t total = rows * width;
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t m = i / width, c = i % width;
+        const float g = to_float(gate[m * gate_stride + c / part]);
+        out[i] = from_float<elem_t>(to_float(x[i]) / (1.0f + expf(-g)));
+    }
+}
+
 static int grid_for(size_t count, int block) {
     size_t g = (count + block - 1) / block;
     return (int)(g > 65535 ? 65535 : (g == 0 ? 1 : g));
@@ -921,6 +1004,61 @@ int mlr_relu_squared(const void* x, void* out, size_t count, hipStream_t stream)
 int mlr_cast_rows(const float* h, void* out, size_t count, hipStream_t stream) {
     if (count == 0) return 0;
     cast_rows_kernel<<<grid_for(count, 256), 256, 0, stream>>>(h, (elem_t*)out, count);
+    return (int)hipGetLastError();
+}
+
+// out[r] = tanh(alpha (h + delta)[rows[r] or r]) w + b; h += delta when write_h
+int mlr_tanh_norm_rows(float* h, const void* delta, const float* w, const float* b, float alpha, void* out,
+                       const int32_t* rows, int n_out, int width, int write_h, hipStream_t stream) {
+    if (n_out <= 0 || width <= 0) return 0;
+    if (width % 4 == 0)
+        tanh_norm_rows_kernel<4><<<grid_for((size_t)n_out * (width / 4), 256), 256, 0, stream>>>(
+            h, (const elem_t*)delta, w, b, alpha, (elem_t*)out, rows, (size_t)n_out, width, write_h);
+    else
+        tanh_norm_rows_kernel<1><<<grid_for((size_t)n_out * width, 256), 256, 0, stream>>>(
+            h, (const elem_t*)delta, w, b, alpha, (elem_t*)out, rows, (size_t)n_out, width, write_h);
+    return (int)hipGetLastError();
+}
+
+// h += tanh(alpha_a delta) wa + ba (+ extra); out (may be null) = tanh(alpha_n h) wn + bn
+int mlr_tanh_norm_add(const void* delta, const float* wa, const float* ba, float alpha_a, float* h, const float* extra,
+                      const float* wn, const float* bn, float alpha_n, void* out, int rows, int width, hipStream_t stream) {
+    if (rows <= 0 || width <= 0) return 0;
+    if (out != nullptr && (wn == nullptr || bn == nullptr)) return -1;
+    if (width % 4 == 0)
+        tanh_norm_add_kernel<4><<<grid_for((size_t)rows * (width / 4), 256), 256, 0, stream>>>(
+            (const elem_t*)delta, wa, ba, alpha_a, h, extra, wn, bn, alpha_n, (elem_t*)out, (size_t)rows, width);
+    else
+        tanh_norm_add_kernel<1><<<grid_for((size_t)rows * width, 256), 256, 0, stream>>>(
+            (const elem_t*)delta, wa, ba, alpha_a, h, extra, wn, bn, alpha_n, (elem_t*)out, (size_t)rows, width);
+    return (int)hipGetLastError();
+}
+
+int mlr_residual_add_float(float* h, const float* extra, size_t count, hipStream_t stream) {
+    if (count == 0) return 0;
+    residual_add_float_kernel<<<grid_for(count, 256), 256, 0, stream>>>(h, extra, count);
+    return (int)hipGetLastError();
+}
+
+int mlr_copy_float(const float* src, float* dst, size_t count, hipStream_t stream) {
+    if (count == 0) return 0;
+    copy_float_kernel<<<grid_for(count, 256), 256, 0, stream>>>(src, dst, count);
+    return (int)hipGetLastError();
+}
+
+int mlr_tanh_cap(float* x, float cap, size_t count, hipStream_t stream) {
+    if (count == 0) return 0;
+    if (!(cap > 0.f)) return -1;
+    tanh_cap_kernel<<<grid_for(count, 256), 256, 0, stream>>>(x, cap, count);
+    return (int)hipGetLastError();
+}
+
+int mlr_head_gate_mul(const void* x, const void* gate, long gate_stride, void* out, int rows, int width, int part,
+                      hipStream_t stream) {
+    if (rows <= 0 || width <= 0) return 0;
+    if (part < 1 || width % part != 0) return -1;
+    head_gate_mul_kernel<<<grid_for((size_t)rows * width, 256), 256, 0, stream>>>((const elem_t*)x, (const elem_t*)gate,
+                                                                                 gate_stride, (elem_t*)out, (size_t)rows, width, part);
     return (int)hipGetLastError();
 }
 

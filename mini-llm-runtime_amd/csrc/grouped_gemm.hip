@@ -246,13 +246,21 @@ __device__ __forceinline__ void wave_best(float& value, int& index) {
 // equal groups of neighbours; a group's score is the sum of its two largest s (of its only one, when a group is
 // one expert); only experts of the `group_keep` best groups stand; of those the `top` largest s are chosen
 // (ties: the lower index), ids[m][i] in descending order of s with weights[m][i] = s itself.
+// With `correction` [experts] the choice (of groups and of experts) goes by s + correction while the weights stay
+// the plain s; with `renorm` the chosen weights are divided by their sum (+ 1e-20); `out_scale` multiplies them.
 __global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict__ z, int32_t* __restrict__ ids,
                                                          float* __restrict__ weights, int experts, int top,
-                                                         int group_count, int group_keep) {
-    __shared__ float s_lds[MAX_EXPERTS];
+                                                         int group_count, int group_keep,
+                                                         const float* __restrict__ correction, int renorm, float out_scale) {
+    __shared__ float s_lds[MAX_EXPERTS];      // what the choice goes by
+    __shared__ float w_lds[MAX_EXPERTS];      // the plain scores
     __shared__ float g_lds[MAX_EXPERTS];
     const int m = blockIdx.x, lane = threadIdx.x;
-    for (int e = lane; e < experts; e += 64) s_lds[e] = 1.0f / (1.0f + expf(-z[(size_t)m * experts + e]));
+    for (int e = lane; e < experts; e += 64) {
+        const float sc = 1.0f / (1.0f + expf(-z[(size_t)m * experts + e]));
+        w_lds[e] = sc;
+        s_lds[e] = correction != nullptr ? sc + correction[e] : sc;
+    }
     __syncthreads();
     const int per = experts / group_count;
     for (int gidx = lane; gidx < group_count; gidx += 64) {
@@ -294,6 +302,7 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict
             if (e < experts && e / per == which) cand[i] = s_lds[e];
         }
     }
+    float chosen_sum = 0.f;
     for (int round = 0; round < top; ++round) {
         float best = -INFINITY;
         int which = 0x7fffffff;
@@ -310,9 +319,18 @@ __global__ __launch_bounds__(64) void router_topk_kernel(const float* __restrict
 #pragma unroll
         for (int i = 0; i < EXPERT_REGS; ++i)
             if (lane + 64 * i == which) cand[i] = -INFINITY;
+        chosen_sum += w_lds[which];                           // (the same on every lane, in the order of the choices)
         if (lane == 0) {
             ids[(size_t)m * top + round] = which;
-            weights[(size_t)m * top + round] = best;
+            weights[(size_t)m * top + round] = w_lds[which];
+        }
+    }
+    if (renorm || out_scale != 1.0f) {
+        __syncthreads();
+        for (int r = lane; r < top; r += 64) {
+            float w = weights[(size_t)m * top + r];
+            if (renorm) w = w / (chosen_sum + 1e-20f);
+            weights[(size_t)m * top + r] = w * out_scale;
         }
     }
 }
@@ -394,12 +412,13 @@ int mlr_grouped_gemm(const void* a, long lda, long a_group, const void* w, long 
 }
 
 int mlr_router_topk(const float* z, int32_t* ids, float* weights, int rows, int experts, int top, int group_count,
-                    int group_keep, hipStream_t stream) {
+                    int group_keep, const float* correction, int renorm, float out_scale, hipStream_t stream) {
     if (rows <= 0) return 0;
     if (experts < 1 || experts > MAX_EXPERTS || group_count < 1 || experts % group_count != 0 || group_keep < 1 ||
         group_keep > group_count || top < 1 || top > group_keep * (experts / group_count))
         return -1;
-    router_topk_kernel<<<rows, 64, 0, stream>>>(z, ids, weights, experts, top, group_count, group_keep);
+    router_topk_kernel<<<rows, 64, 0, stream>>>(z, ids, weights, experts, top, group_count, group_keep, correction, renorm,
+                                                out_scale);
     return (int)hipGetLastError();
 }
 

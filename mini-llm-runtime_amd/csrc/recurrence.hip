@@ -259,14 +259,20 @@ struct DeltaArgs {
     const elem_t* q; long q_stride;            // q[r * q_stride + (head / heads_per_group) * N + i], as projected
     const elem_t* k; long k_stride;
     const elem_t* v; long v_stride;            // v[r * v_stride + head * V + j]
-    const float* log_decay;                    // [rows][heads * N]
+    const float* log_decay;                    // [rows][heads * N], or with decay_per_head [rows][heads]
     const float* beta_raw; long beta_stride;   // beta = sigmoid(beta_raw[r * stride + head])
     float* out;                                // [rows, heads * V]
     const float* live; float* stage; long state_stride;     // a request's S as [heads][N][V]
     const int32_t* seg_first; const int32_t* seg_count; const int32_t* slots;
     int heads, heads_per_group, N, V, write_state, unit_norm;
     float q_scale, unit_eps;
+    int decay_per_head;                        // one decay for all key channels of a head
 };
+
+// Where the log decay of (row, head, key channel i) lies.
+__device__ __forceinline__ size_t decay_at(const DeltaArgs& a, size_t row, int head, int i) {
+    return a.decay_per_head ? row * (size_t)a.heads + head : row * ((size_t)a.heads * a.N) + (size_t)head * a.N + i;
+}
 
 #define DELTA_TILE 16
 
@@ -310,7 +316,7 @@ __global__ __launch_bounds__(64) void delta_rule_kernel(DeltaArgs a) {
                 if (i < N) {
                     dq = to_float(a.q[row * a.q_stride + qk_head * N + i]);
                     dk = to_float(a.k[row * a.k_stride + qk_head * N + i]);
-                    dg = expf(a.log_decay[row * ((size_t)a.heads * N) + head * N + i]);
+                    dg = expf(a.log_decay[decay_at(a, row, head, i)]);
                 }
                 qq += dq * dq;
                 kk += dk * dk;
@@ -424,7 +430,7 @@ __global__ __launch_bounds__(256) void delta_chunk_prepare_kernel(DeltaChunkArgs
             const size_t row = (size_t)(r0 + t);
             dq = to_float(a.q[row * a.q_stride + qk_head * N + i]);
             dk = to_float(a.k[row * a.k_stride + qk_head * N + i]);
-            dc = a.log_decay[row * ((size_t)a.heads * N) + head * N + i];
+            dc = a.log_decay[decay_at(a, row, head, i)];
         }
         q_l[t * NS + i] = dq; k_l[t * NS + i] = dk; c_l[t * NS + i] = dc;
     }
@@ -735,14 +741,14 @@ int mlr_delta_rule(const void* q, long q_stride, const void* k, long k_stride, c
                    const float* log_decay, const float* beta_raw, long beta_stride, float* out, const float* live, float* stage,
                    long state_stride, const int32_t* seg_first, const int32_t* seg_count, const int32_t* slots, int segments,
                    int heads, int heads_per_group, int n_keys, int n_values, int write_state, int unit_norm, float q_scale,
-                   float unit_eps, hipStream_t stream) {
+                   float unit_eps, int decay_per_head, hipStream_t stream) {
     if (segments <= 0) return 0;
     if (n_keys < 1 || n_keys > 256 || n_values < 1 || heads < 1 || heads > 65535 || heads_per_group < 1 ||
         heads % heads_per_group)
         return -1;
     DeltaArgs a{(const elem_t*)q, q_stride, (const elem_t*)k, k_stride, (const elem_t*)v, v_stride, log_decay, beta_raw,
                 beta_stride, out, live, stage, state_stride, seg_first, seg_count, slots, heads, heads_per_group, n_keys,
-                n_values, write_state, unit_norm, q_scale, unit_eps};
+                n_values, write_state, unit_norm, q_scale, unit_eps, decay_per_head};
     int parts = n_keys > 128 ? 4 : n_keys > 64 ? 2 : 1;
     if (n_values <= 16 && parts < 4) parts = 4;
     else if (n_values <= 32 && parts < 2) parts = 2;
@@ -772,14 +778,14 @@ int mlr_delta_rule_chunked(const void* q, long q_stride, const void* k, long k_s
                            float* stage, long state_stride, const int32_t* seg_first, const int32_t* seg_count,
                            const int32_t* slots, int segments, const int32_t* chunk_first, const int32_t* chunk_count, int chunks,
                            float* scratch, int heads, int heads_per_group, int n_keys, int n_values, int write_state,
-                           int unit_norm, float q_scale, float unit_eps, hipStream_t stream) {
+                           int unit_norm, float q_scale, float unit_eps, int decay_per_head, hipStream_t stream) {
     if (segments <= 0 || chunks <= 0) return 0;
     if (n_keys < 1 || n_keys > 128 || n_values < 1 || heads < 1 || heads > 65535 || heads_per_group < 1 ||
         heads % heads_per_group || scratch == nullptr)
         return -1;
     DeltaChunkArgs g{{(const elem_t*)q, q_stride, (const elem_t*)k, k_stride, (const elem_t*)v, v_stride, log_decay, beta_raw,
                       beta_stride, out, live, stage, state_stride, seg_first, seg_count, slots, heads, heads_per_group, n_keys,
-                      n_values, write_state, unit_norm, q_scale, unit_eps},
+                      n_values, write_state, unit_norm, q_scale, unit_eps, decay_per_head},
                      chunk_first, chunk_count, scratch};
     const int C = DELTA_CHUNK, NS = n_keys + 1;
     const size_t lds1 = sizeof(float) * ((size_t)3 * C * NS + (size_t)3 * C * (C + 1) + C);

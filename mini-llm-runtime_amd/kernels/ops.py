@@ -214,6 +214,14 @@ class Kernels:
         fn = self._lib("elementwise").mlr_residual_add
         _ok(fn(_p(h), _p(delta), _c_size_t(h.numel()), _stream()), "residual_add")
 
+    @timed("norm", _tensors_work())
+    def residual_add_float(self, h, extra):
+        """h += extra, both float (the embedding's output joining the stream again)."""
+        _tensor(h, "h", torch.float32, ndim=2)
+        _tensor(extra, "extra", torch.float32, tuple(h.shape))
+        _ok(self._lib("elementwise").mlr_residual_add_float(_p(h), _p(extra), _c_size_t(h.numel()), _stream()),
+            "residual_add_float")
+
     @timed("activation", _tensors_work())
     def silu_mul(self, gate_up, act):
         """act[m, f] = silu(gate_up[m, f]) * gate_up[m, F + f]."""
@@ -951,11 +959,13 @@ class Kernels:
 
     @timed("recurrence", _tensors_work())
     def delta_rule(self, q, k, v, log_decay, beta_raw, out, live, stage, state_offset, seg_first, seg_count, segments, slots,
-                   heads, n_keys, n_values, heads_per_group=1, q_scale=1.0, unit_norm=True, unit_eps=1e-6, write_state=True):
+                   heads, n_keys, n_values, heads_per_group=1, q_scale=1.0, unit_norm=True, unit_eps=1e-6, write_state=True,
+                   decay_per_head=False):
         """Per request of the step and head, from the live state: S <- diag(exp(log_decay_t)) S; u = beta_t (v_t - S^T k_t);
         S <- S + k_t u^T; out_t = S^T q_t, with beta = sigmoid(beta_raw).  q, k: columns [rows, (heads / heads_per_group) *
         n_keys], made unit vectors per head inside (x / sqrt(sum x^2 + unit_eps); `unit_norm` False: taken as they
-        are) and q multiplied by q_scale; v: columns [rows, heads * n_values]; log_decay float [rows, heads * n_keys];
+        are) and q multiplied by q_scale; v: columns [rows, heads * n_values]; log_decay float [rows, heads * n_keys], or
+        with `decay_per_head` [rows, heads] (one decay for all key channels of a head);
         beta_raw float columns [rows, heads]; the state [heads][n_keys][n_values] floats from `state_offset` on in a
         slot's row of `live`/`stage`."""
         rows = v.shape[0]
@@ -965,7 +975,7 @@ class Kernels:
         qs = self._columns(q, "q", self.dtype, rows, groups * n_keys)
         ks = self._columns(k, "k", self.dtype, rows, groups * n_keys)
         vs = self._columns(v, "v", self.dtype, rows, heads * n_values)
-        _tensor(log_decay, "log_decay", torch.float32, (rows, heads * n_keys))
+        _tensor(log_decay, "log_decay", torch.float32, (rows, heads if decay_per_head else heads * n_keys))
         bs = self._columns(beta_raw, "beta_raw", torch.float32, rows, heads)
         _tensor(out, "out", torch.float32, (rows, heads * n_values))
         self._check_state(live, stage, state_offset, heads * n_keys * n_values)
@@ -979,7 +989,7 @@ class Kernels:
             ctypes.c_long(bs), _p(out), _ptr(live.data_ptr() + at), _ptr(stage.data_ptr() + at), ctypes.c_long(live.stride(0)),
             _p(seg_first), _p(seg_count), _p(slots), _c_int(segments), _c_int(heads), _c_int(heads_per_group), _c_int(n_keys),
             _c_int(n_values), _c_int(1 if write_state else 0), _c_int(1 if unit_norm else 0), _c_float(q_scale),
-            _c_float(unit_eps), _stream()), "delta_rule")
+            _c_float(unit_eps), _c_int(1 if decay_per_head else 0), _stream()), "delta_rule")
 
     DELTA_CHUNK_MAX_KEYS = 128
 
@@ -996,7 +1006,7 @@ class Kernels:
     @timed("recurrence", _tensors_work())
     def delta_rule_chunked(self, q, k, v, log_decay, beta_raw, out, live, stage, state_offset, seg_first, seg_count, segments,
                            slots, chunk_first, chunk_count, chunks, scratch, heads, n_keys, n_values, heads_per_group=1,
-                           q_scale=1.0, unit_norm=True, unit_eps=1e-6, write_state=True):
+                           q_scale=1.0, unit_norm=True, unit_eps=1e-6, write_state=True, decay_per_head=False):
         """`delta_rule` over chunks of tokens: `chunk_first`/`chunk_count` cut every request of the step into chunks of
         at most `delta_chunk_tokens()` tokens (a request's chunks one after the other, the requests in the order of
         `seg_first`); what a chunk does to ANY state it might start from is worked out for all chunks side by side,
@@ -1009,7 +1019,7 @@ class Kernels:
         qs = self._columns(q, "q", self.dtype, rows, groups * n_keys)
         ks = self._columns(k, "k", self.dtype, rows, groups * n_keys)
         vs = self._columns(v, "v", self.dtype, rows, heads * n_values)
-        _tensor(log_decay, "log_decay", torch.float32, (rows, heads * n_keys))
+        _tensor(log_decay, "log_decay", torch.float32, (rows, heads if decay_per_head else heads * n_keys))
         bs = self._columns(beta_raw, "beta_raw", torch.float32, rows, heads)
         _tensor(out, "out", torch.float32, (rows, heads * n_values))
         self._check_state(live, stage, state_offset, heads * n_keys * n_values)
@@ -1027,8 +1037,8 @@ class Kernels:
             ctypes.c_long(bs), _p(out), _ptr(live.data_ptr() + at), _ptr(stage.data_ptr() + at), ctypes.c_long(live.stride(0)),
             _p(seg_first), _p(seg_count), _p(slots), _c_int(segments), _p(chunk_first), _p(chunk_count), _c_int(chunks),
             _p(scratch), _c_int(heads), _c_int(heads_per_group), _c_int(n_keys), _c_int(n_values),
-            _c_int(1 if write_state else 0), _c_int(1 if unit_norm else 0), _c_float(q_scale), _c_float(unit_eps), _stream()),
-            "delta_rule_chunked")
+            _c_int(1 if write_state else 0), _c_int(1 if unit_norm else 0), _c_float(q_scale), _c_float(unit_eps),
+            _c_int(1 if decay_per_head else 0), _stream()), "delta_rule_chunked")
 
     # -- differential attention -----------------------------------------------------------------------
     DIFF_MAX_HEAD_DIM = 256
@@ -1056,6 +1066,34 @@ class Kernels:
                _c_int(block_table.shape[1]), _p(slots), _p(positions), _c_int(rows), _c_int(kv_heads), _c_int(2 * head_dim),
                _c_int(value_dim), _c_int(page_size), _stream()), "diff_kv_write")
 
+    @timed("rope_kv", _tensors_work())
+    def diff_qkv_prep(self, q, k, v, k_pages, v_pages, block_table, slots, positions, rope, q_heads, kv_heads, head_dim,
+                      value_dim, page_size, write_cache=True, interleaved=False):
+        """The step's queries and keys (both maps of every head) turned by their positions, the keys and values into
+        their pages.  q: columns [rows, q_heads * 2 * head_dim], turned in place; rope float [positions, rot] (cosines,
+        then sines): the first rot channels of each map turn, in pairs (j, j + rot / 2) or, `interleaved`,
+        (2 j, 2 j + 1); None: nothing turns."""
+        rows = k.shape[0]
+        qs = self._columns(q, "q", self.dtype, rows, q_heads * 2 * head_dim)
+        ks = self._columns(k, "k", self.dtype, rows, kv_heads * 2 * head_dim)
+        vs = self._columns(v, "v", self.dtype, rows, kv_heads * value_dim)
+        self._check_diff_cache(k_pages, v_pages, kv_heads, head_dim, value_dim, page_size)
+        _tensor(block_table, "block_table", torch.int32, ndim=2)
+        _tensor(slots, "slots", torch.int32, (rows,))
+        _tensor(positions, "positions", torch.int32, (rows,))
+        rot = 0
+        if rope is not None:
+            _tensor(rope, "rope", torch.float32, ndim=2)
+            rot = rope.shape[1]
+            _need(rot % 2 == 0 and 2 <= rot <= head_dim, "diff_qkv_prep: the rotation turns an even part of a map")
+        fn = self._lib("diff_attention").mlr_diff_qkv_prep
+        _ok(fn(_p(q), ctypes.c_long(qs), _p(k), ctypes.c_long(ks), _p(v), ctypes.c_long(vs), _p(k_pages), _p(v_pages),
+               _p(block_table), _c_int(block_table.shape[1]), _p(slots), _p(positions), _p(rope), _c_int(rot),
+               _c_int(1 if interleaved else 0), _c_int(rows), _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim),
+               _c_int(value_dim), _c_int(page_size), _c_int(1 if write_cache else 0), _stream()), "diff_qkv_prep")
+
+    MASK_KINDS = {None: 0, "window": 1, "chunk": 2}
+
     @staticmethod
     def diff_partial_numel(rows, q_heads, value_dim, max_splits):
         return rows * q_heads * 2 * max(1, max_splits) * (value_dim + 2)
@@ -1063,10 +1101,12 @@ class Kernels:
     @timed("attention")
     def diff_attention(self, q, k_pages, v_pages, block_table, slots, positions, gate, out, partial, q_heads, kv_heads,
                        head_dim, value_dim, page_size, scale, lam, out_scale, eps, softcap=None, temp_coef=0.0,
-                       temp_every=1.0, split_keys=0, max_splits=1):
+                       temp_every=1.0, split_keys=0, max_splits=1, mask=None, mask_size=0):
         """Differential attention of every token of the step over the cached keys at positions <= its own (the step's
         own keys are in the cache already): out [rows, q_heads * value_dim], normed, scaled and gated by
-        sigmoid(gate) (gate None: no gate).  q: columns [rows, q_heads * 2 * head_dim]."""
+        sigmoid(gate) (gate None: no gate).  q: columns [rows, q_heads * 2 * head_dim].  `mask`: None, or "window"
+        (the last mask_size positions) or "chunk" (the query's own block of mask_size positions)."""
+        _need(mask in self.MASK_KINDS and (mask is None or mask_size >= 1), "diff_attention: mask rule")
         rows = q.shape[0]
         qs = self._columns(q, "q", self.dtype, rows, q_heads * 2 * head_dim)
         gs = self._columns(gate, "gate", self.dtype, rows, q_heads * value_dim) if gate is not None else 0
@@ -1089,7 +1129,8 @@ class Kernels:
                _p(positions), _p(gate), ctypes.c_long(gs), _p(out), _p(partial), _c_int(rows), _c_int(q_heads),
                _c_int(kv_heads), _c_int(head_dim), _c_int(value_dim), _c_int(page_size), _c_float(scale),
                _c_float(softcap or 0.0), _c_float(temp_coef), _c_float(temp_every), _c_float(lam), _c_float(out_scale),
-               _c_float(eps), _c_int(split_keys), _c_int(max_splits), _ptr(0), _ptr(0), _c_int(0), _c_int(0), _stream()),
+               _c_float(eps), _c_int(split_keys), _c_int(max_splits), _ptr(0), _ptr(0), _c_int(0), _c_int(0),
+               _c_int(self.MASK_KINDS[mask]), _c_int(mask_size), _stream()),
             "diff_attention")
 
     def diff_tiles_supported(self, q_heads, kv_heads, head_dim, value_dim, page_size, q_stride=0, gate_stride=0):
@@ -1116,7 +1157,7 @@ class Kernels:
     def diff_attention_tiles(self, q, k_pages, v_pages, block_table, slots, positions, gate, out, partial, group_row0,
                              group_ntok, groups, group_tokens, q_heads, kv_heads, head_dim, value_dim, page_size, scale, lam,
                              out_scale, eps, softcap=None, temp_coef=0.0, temp_every=1.0, split_keys=0, max_splits=1,
-                             max_context=None):
+                             max_context=None, mask=None, mask_size=0):
         """As `diff_attention` for the rows of `groups` groups of consecutive tokens of one request each (first row,
         number of tokens: device int32 vectors; at most `group_tokens` tokens a group), on the matrix cores.
         `max_context`: a bound on the step's positions + 1 (default: what the block table can hold); the keys that one
@@ -1149,7 +1190,9 @@ class Kernels:
         _need(kv_heads * 4 <= 65535 and max_splits <= 65535, "diff_attention_tiles: grid too large")
         if max_context is None:
             max_context = block_table.shape[1] * page_size
-        _need(self.diff_tiles_reach(page_size) >= (split_keys if max_splits > 1 else max_context),
+        _need(mask in self.MASK_KINDS and (mask is None or mask_size >= 1), "diff_attention_tiles: mask rule")
+        walk = max_context if mask is None else min(max_context, mask_size + group_tokens + 2 * ATTENTION_TILE_KEYS)
+        _need(self.diff_tiles_reach(page_size) >= (split_keys if max_splits > 1 else walk),
               "diff_attention_tiles: one workgroup would walk more pages than it keeps ids of; cut the keys into ranges")
         fn = self._lib("diff_attention").mlr_diff_attention_tiles
         _ok(fn(_p(q), ctypes.c_long(qs), _p(k_pages), _p(v_pages), _p(block_table), _c_int(block_table.shape[1]), _p(slots),
@@ -1157,7 +1200,8 @@ class Kernels:
                _p(group_ntok), _c_int(groups), _c_int(group_tokens), _c_int(q_heads), _c_int(kv_heads), _c_int(head_dim),
                _c_int(value_dim), _c_int(page_size), _c_float(scale), _c_float(softcap or 0.0), _c_float(temp_coef),
                _c_float(temp_every), _c_float(lam), _c_float(out_scale), _c_float(eps), _c_int(split_keys),
-               _c_int(max_splits), _c_int(max_context), _stream()), "diff_attention_tiles")
+               _c_int(max_splits), _c_int(max_context), _c_int(self.MASK_KINDS[mask]), _c_int(mask_size), _stream()),
+            "diff_attention_tiles")
 
     # -- layer norm, plain activations ---------------------------------------------------------
     @timed("norm", _tensors_work())
@@ -1175,6 +1219,75 @@ class Kernels:
         _ok(self._lib("elementwise").mlr_layernorm(_p(delta), _ptr(0), _p(weight), _p(bias), _ptr(0), _p(h), _p(cast),
                                                    _ptr(0), _c_int(m), _c_int(width), _c_float(eps), _c_float(1.0),
                                                    _stream()), "layernorm_add")
+
+    @timed("norm", _tensors_work())
+    def tanh_norm_rows(self, h, delta, weight, bias, alpha, out, rows=None, write_h=True):
+        """x = h + delta (delta may be None; written back to h when write_h); out[r] = T(tanh(alpha x[rows[r] or r]) *
+        weight + bias): a norm that takes no statistics, element by element in 32-bit."""
+        _tensor(h, "h", torch.float32, ndim=2)
+        m, width = h.shape
+        if delta is not None:
+            _tensor(delta, "delta", self.dtype, (m, width))
+        _tensor(weight, "weight", torch.float32, (width,))
+        _tensor(bias, "bias", torch.float32, (width,))
+        if rows is not None:
+            _tensor(rows, "rows", torch.int32, ndim=1)
+            _need(delta is None or not write_h, "tanh_norm_rows: a gathered norm does not write the stream")
+        n_out = rows.numel() if rows is not None else m
+        _tensor(out, "out", self.dtype, (n_out, width))
+        _ok(self._lib("elementwise").mlr_tanh_norm_rows(_p(h), _p(delta), _p(weight), _p(bias), _c_float(alpha), _p(out),
+                                                        _p(rows), _c_int(n_out), _c_int(width), _c_int(1 if write_h else 0),
+                                                        _stream()), "tanh_norm_rows")
+
+    @timed("norm", _tensors_work())
+    def tanh_norm_add(self, delta, weight, bias, alpha, h, extra=None, then=None, out=None):
+        """h += tanh(alpha delta) * weight + bias (+ extra, float like h): the norm of what a sublayer gave, added to the
+        float residual stream; `then` = (weight, bias, alpha) of the norm in front of the next sublayer and `out` (the
+        engine's element type): out = that norm of the new h, in the same pass."""
+        _tensor(h, "h", torch.float32, ndim=2)
+        m, width = h.shape
+        _tensor(delta, "delta", self.dtype, (m, width))
+        _tensor(weight, "weight", torch.float32, (width,))
+        _tensor(bias, "bias", torch.float32, (width,))
+        if extra is not None:
+            _tensor(extra, "extra", torch.float32, (m, width))
+        wn = bn = None
+        an = 0.0
+        if out is not None:
+            _need(then is not None, "tanh_norm_add: an output needs the norm that makes it")
+            wn, bn, an = then
+            _tensor(wn, "then.weight", torch.float32, (width,))
+            _tensor(bn, "then.bias", torch.float32, (width,))
+            _tensor(out, "out", self.dtype, (m, width))
+        _ok(self._lib("elementwise").mlr_tanh_norm_add(_p(delta), _p(weight), _p(bias), _c_float(alpha), _p(h), _p(extra),
+                                                       _p(wn), _p(bn), _c_float(an), _p(out), _c_int(m), _c_int(width),
+                                                       _stream()), "tanh_norm_add")
+
+    @timed("norm", _tensors_work())
+    def copy_float(self, src, dst):
+        """dst = src (float tensors of one shape)."""
+        _tensor(src, "src", torch.float32)
+        _tensor(dst, "dst", torch.float32, tuple(src.shape))
+        _ok(self._lib("elementwise").mlr_copy_float(_p(src), _p(dst), _c_size_t(src.numel()), _stream()), "copy_float")
+
+    @timed("activation", _tensors_work())
+    def tanh_cap(self, x, cap):
+        """x <- cap * tanh(x / cap) on float values in place (a cap on logits)."""
+        _tensor(x, "x", torch.float32)
+        _need(cap > 0.0, "tanh_cap: the cap must be positive")
+        _ok(self._lib("elementwise").mlr_tanh_cap(_p(x), _c_float(cap), _c_size_t(x.numel()), _stream()), "tanh_cap")
+
+    @timed("activation", _tensors_work())
+    def head_gate_mul(self, x, gate, out, heads):
+        """out[m, head, :] = x[m, head, :] * sigmoid(gate[m, head]): x, out [rows, heads * part]; gate: columns
+        [rows, heads] of a row-major matrix; out may be x."""
+        _tensor(x, "x", self.dtype, ndim=2)
+        m, width = x.shape
+        _need(heads >= 1 and width % heads == 0, "head_gate_mul: the width is no multiple of the heads")
+        stride = self._columns(gate, "gate", self.dtype, m, heads)
+        _tensor(out, "out", self.dtype, (m, width))
+        _ok(self._lib("elementwise").mlr_head_gate_mul(_p(x), _p(gate), ctypes.c_long(stride), _p(out), _c_int(m),
+                                                       _c_int(width), _c_int(width // heads), _stream()), "head_gate_mul")
 
     @timed("norm", _tensors_work())
     def layernorm_rows(self, h, weight, bias, out, eps, rows=None, out_scale=1.0):
@@ -1444,10 +1557,14 @@ class Kernels:
             _c_int(self.GROUPED_ACTS[act]), _c_int(0), _stream()), "experts_gemm")
 
     @timed("activation", _tensors_work())
-    def router_topk(self, logits, ids, weights, group_count, group_keep):
+    def router_topk(self, logits, ids, weights, group_count=1, group_keep=1, correction=None, renormalize=False, scale=1.0):
         """Per row of the router logits [rows, experts] (float): s = sigmoid(z); of the group_count equal groups of
         neighbouring experts the group_keep with the largest sum of their two best s stay; ids [rows, top] int32 the
-        experts with the largest s among those, weights [rows, top] float their s."""
+        experts with the largest s among those, weights [rows, top] float their s.  With `correction` (float
+        [experts]) every choice goes by s + correction and the weights stay s; `renormalize`: the chosen weights over
+        their sum (+ 1e-20); `scale` multiplies them."""
+        if correction is not None:
+            _tensor(correction, "correction", torch.float32, (logits.shape[1],))
         _tensor(logits, "logits", torch.float32, ndim=2)
         rows, experts = logits.shape
         _tensor(ids, "ids", torch.int32, ndim=2)
@@ -1458,7 +1575,8 @@ class Kernels:
               and 1 <= group_keep <= group_count and 1 <= top <= group_keep * (experts // group_count),
               "router_topk: experts up to 256 in equal groups, and no more choices than the kept groups hold")
         _ok(self._lib("grouped_gemm").mlr_router_topk(_p(logits), _p(ids), _p(weights), _c_int(rows), _c_int(experts),
-                                                      _c_int(top), _c_int(group_count), _c_int(group_keep), _stream()),
+                                                      _c_int(top), _c_int(group_count), _c_int(group_keep), _p(correction),
+                                                      _c_int(1 if renormalize else 0), _c_float(scale), _stream()),
             "router_topk")
 
     @timed("gemm")

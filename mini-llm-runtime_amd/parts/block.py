@@ -1,7 +1,9 @@
 """Arrangement of the parts in a layer.  Pre-norm residual block (src/minillm/runtime.cpp:245-337):
 h += mixer(norm1(h)); h += ffn(norm2(h)).  The residual stream h is float; every add into it is
 fused with the norm that follows, so a block hands its last output on as `pending` instead of
-adding it itself.  `norm2` and `ffn` may be missing: a layer of the first sublayer only."""
+adding it itself.  `norm2` and `ffn` may be missing: a layer of the first sublayer only.
+Other arrangements: mixer and feed-forward side by side (`parallel`), norms behind the sublayers (`postnorm`), norms in
+front of AND behind each sublayer (`sandwich`)."""
 from __future__ import annotations
 
 from .registry import Complete, Handoff, build_part, register_part
@@ -177,3 +179,74 @@ class PostNormBlock:
             fed = self.ffn.forward(ctx, x)
             self.norm2.add_into(ctx, fed, h, cast=x if narrow and next_norm is not None else None)
         return Streamed(x) if next_norm is not None else None
+
+
+@register_part("block", "sandwich")
+class SandwichBlock:
+    """A norm in front of and one behind each sublayer: h += norm1_after(mixer(norm1(h))); h += norm2_after(ffn(norm2(h))).
+    The norm behind a sublayer, the residual sum and the norm in front of the next sublayer are one pass over the
+    stream where the norms can (`add_into(..., then=, out=)`: the norm without statistics); `norm2`, `ffn` and
+    `norm2_after` may be missing.  `extra` (a float matrix like h) is added to the stream with the block's last
+    sublayer, before the next block's norm."""
+    graph_safe = True
+    adds_extra = True
+
+    def __init__(self, spec):
+        self.norm1 = build_part("norm", spec.norm1)
+        self.mixer = build_part("mixer", spec.mixer)
+        if spec.norm1_after is None:
+            raise ValueError("a sandwich block needs the norm behind its mixer")
+        self.norm1_after = build_part("norm", spec.norm1_after)
+        if not ((spec.ffn is None) == (spec.norm2 is None) == (spec.norm2_after is None)):
+            raise ValueError("a sandwich block has a feed-forward and both its norms, or none of the three")
+        self.norm2 = build_part("norm", spec.norm2) if spec.norm2 is not None else None
+        self.ffn = build_part("ffn", spec.ffn) if spec.ffn is not None else None
+        self.norm2_after = build_part("norm", spec.norm2_after) if spec.norm2_after is not None else None
+        for norm in (self.norm1_after, self.norm2_after):
+            if norm is not None and not hasattr(norm, "add_into"):
+                raise ValueError("a sandwich block needs norms behind its sublayers that can add into the stream (`add_into`)")
+
+    def parts(self):
+        out = {"norm1": self.norm1, "mixer": self.mixer, "norm1_after": self.norm1_after}
+        if self.ffn is not None:
+            out.update(norm2=self.norm2, ffn=self.ffn, norm2_after=self.norm2_after)
+        return out
+
+    def workspace_plan(self, rows, dtype, limits):
+        return {("normed", dtype): rows * self.norm1.size}
+
+    @staticmethod
+    def _same_pass(after, then):
+        """Whether `after.add_into` can take the norm `then` in its pass: both of one kind that offers it."""
+        return then is not None and type(then) is type(after) and hasattr(then, "params")
+
+    def forward(self, ctx, h, pending, cache_id, write_cache=True, next_norm=None, extra=None):
+        from .registry import Normed
+        normed = ctx.workspace.get("normed", tuple(h.shape), ctx.dtype)
+        if isinstance(pending, Normed) and pending.norms == (self.norm1,):
+            x = pending.outputs[0]                       # the block before normed the stream for this one
+        else:
+            self.norm1.forward(ctx, h, None if isinstance(pending, Complete) else pending, normed)
+            x = normed
+        mixed = self.mixer.forward(ctx, x, cache_id, write_cache)
+        if self.ffn is None:
+            return self._last(ctx, h, mixed, self.norm1_after, next_norm, extra, normed)
+        if self._same_pass(self.norm1_after, self.norm2):
+            self.norm1_after.add_into(ctx, mixed, h, then=self.norm2, out=normed)
+        else:
+            self.norm1_after.add_into(ctx, mixed, h)
+            self.norm2.forward(ctx, h, None, normed)
+        fed = self.ffn.forward(ctx, normed)
+        return self._last(ctx, h, fed, self.norm2_after, next_norm, extra, normed)
+
+    def _last(self, ctx, h, delta, after, next_norm, extra, normed):
+        """The block's last sublayer into the stream; the next block's first norm in the same pass where it can be."""
+        from .registry import Normed
+        if self._same_pass(after, next_norm) and next_norm.size == h.shape[1]:
+            after.add_into(ctx, delta, h, extra=extra, then=next_norm, out=normed)
+            return Normed((next_norm,), (normed,))
+        if extra is not None:
+            after.add_into(ctx, delta, h, extra=extra)
+        else:
+            after.add_into(ctx, delta, h)
+        return None

@@ -3,8 +3,10 @@ queries and keys of their own over the same values; the head's output is map 1 -
 lam = exp(lq1 . lk1) - exp(lq2 . lk2) + lam_init (one number a layer), divided by its root mean square over the
 value channels, times `out_scale`, times sigmoid of the head's gate; then the output projection.  Query and key
 channels of a map (`head_dim`) and value channels (`value_dim`) are sizes of their own; consecutive query heads
-share a kv head.  There is no rotation: a query's position enters as a factor on it
-(`QueryTemperature`), a score is squashed by `softcap * tanh(score / softcap)`, and position p sees keys 0..p.
+share a kv head.  A query's position may enter as a factor on it (`QueryTemperature`) and a score may be squashed by
+`softcap * tanh(score / softcap)`; with a position part, the first channels of every map of q and k are turned by
+the token's position before the keys are cached; position p sees keys 0..p, or what a mask rule leaves of them
+(the last `size` positions, or the positions of p's own block of `size`).
 
 Per token the cache keeps the keys of both maps [kv_heads, 2 * head_dim] and the values [kv_heads, value_dim]
 (`PagedSpec`).  q, k, v and the gate are one stacked projection of the mixer's input.
@@ -20,7 +22,8 @@ import torch
 
 from ..cache.manager import PAGE, PagedSpec
 from ..weights.loader import WeightSpec, stacked
-from .registry import PartError, register_part
+from .registry import PartError, build_part, register_part
+from .sink_attention import _mask_of, _rope_table
 
 PARTIAL_CAP = 32 << 20        # floats that the key ranges' partial results of one launch may take at most
 SMALL_GROUP = 4               # tokens: a request that brings more of them to a step is a prompt portion
@@ -38,6 +41,8 @@ class DiffAttention:
             raise PartError(f"head_dim {s.head_dim} / value_dim {s.value_dim}: the attention kernels take sizes up to 256")
         if s.gate not in (None, "sigmoid"):
             raise PartError(f"gate {s.gate!r} is not built (sigmoid or none)")
+        self.mask, self.mask_size = _mask_of(s) if getattr(s, "mask", None) is not None else (None, 0)
+        self.position = build_part("position", s.position) if getattr(s, "position", None) is not None else None
         self.q_width, self.k_width = s.q_heads * 2 * s.head_dim, s.kv_heads * 2 * s.head_dim
         self.v_width, self.o_width = s.kv_heads * s.value_dim, s.q_heads * s.value_dim
         self.proj = self.o = None
@@ -71,7 +76,8 @@ class DiffAttention:
     def cache_spec(self):
         s = self.spec
         # (values transposed within a page: the keys of one channel side by side, as the matrix cores want them)
-        return PagedSpec((("k", (s.kv_heads, PAGE, 2 * s.head_dim)), ("v", (s.kv_heads, s.value_dim, PAGE))), None)
+        return PagedSpec((("k", (s.kv_heads, PAGE, 2 * s.head_dim)), ("v", (s.kv_heads, s.value_dim, PAGE))),
+                         self.mask_size if self.mask is not None else None)
 
     def libraries(self):
         return ["gemm", "diff_attention"]
@@ -109,6 +115,8 @@ class DiffAttention:
         s = self.spec
         base, longest = ctx.split_keys, ctx.max_context
         reach = ctx.kernels.diff_tiles_reach(self._page_size)       # the most keys one workgroup walks
+        if self.mask is not None and self.mask_size + 64 + 128 <= reach:
+            return 0, 1                           # (behind a mask a workgroup walks its tokens' window or block only)
         forced = longest > reach
         if base <= 0 and forced:
             raise PartError(f"a context of {longest} tokens needs key ranges (split_keys > 0): one workgroup walks {reach} keys")
@@ -149,7 +157,7 @@ class DiffAttention:
                                    s.value_dim, view.page_size, float(s.scale), self.lam, float(s.out_scale), float(s.eps),
                                    softcap=s.softcap, temp_coef=temp.coef if temp else 0.0,
                                    temp_every=temp.every if temp else 1.0, split_keys=split_keys, max_splits=splits,
-                                   max_context=ctx.max_context)
+                                   max_context=ctx.max_context, mask=self.mask, mask_size=self.mask_size)
 
     def forward(self, ctx, x, cache_id, write_cache=True):
         s = self.spec
@@ -164,7 +172,11 @@ class DiffAttention:
         gate = proj[:, c:] if s.gate is not None else None
         view = ctx.cache.paged_view(cache_id)
         k_pages, v_pages = view.tensors["k"], view.tensors["v"]
-        if write_cache:
+        if self.position is not None:
+            rope, interleaved = _rope_table(self.position, ctx, x.device, s.head_dim)
+            k.diff_qkv_prep(q, keys, values, k_pages, v_pages, view.block_table, ctx.slots, ctx.positions, rope, s.q_heads,
+                            s.kv_heads, s.head_dim, s.value_dim, view.page_size, write_cache, interleaved=interleaved)
+        elif write_cache:
             k.diff_kv_write(keys, values, k_pages, v_pages, view.block_table, ctx.slots, ctx.positions, s.kv_heads,
                             s.head_dim, s.value_dim, view.page_size)
         attn = ctx.workspace.get("attn", (m, self.o_width), x.dtype)
@@ -185,7 +197,8 @@ class DiffAttention:
                              gate[r0:r1] if gate is not None else None, attn[r0:r1], partial, s.q_heads, s.kv_heads,
                              s.head_dim, s.value_dim, view.page_size, float(s.scale), self.lam, float(s.out_scale),
                              float(s.eps), softcap=s.softcap, temp_coef=temp.coef if temp else 0.0,
-                             temp_every=temp.every if temp else 1.0, split_keys=split_keys, max_splits=splits)
+                             temp_every=temp.every if temp else 1.0, split_keys=split_keys, max_splits=splits,
+                             mask=self.mask, mask_size=self.mask_size)
         out = ctx.workspace.get("mixer_out", (m, s.hidden), x.dtype)
         k.gemm(attn, self.o, out)
         return out

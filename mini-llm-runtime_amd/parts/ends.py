@@ -13,7 +13,7 @@ from ..config.specs import EmbedSpec, HeadSpec
 from ..weights.loader import WeightSpec
 from .registry import PartError, register_part
 
-__all__ = ["TokenEmbedding", "PairEmbedding", "LinearHead", "ScaledHead", "EmbedSpec", "HeadSpec"]
+__all__ = ["TokenEmbedding", "PairEmbedding", "LinearHead", "ScaledHead", "CappedHead", "EmbedSpec", "HeadSpec"]
 
 
 @register_part("embed", "token_embedding")
@@ -130,4 +130,18 @@ class ScaledHead(LinearHead):
         logits = super().forward(ctx, final)
         if self.spec.scale != 1.0:
             ctx.kernels.scale_float(logits, float(self.spec.scale))
+        return logits
+
+
+@register_part("head", "capped_head")
+class CappedHead(LinearHead):
+    """logits <- softcap * tanh(logits / softcap) on the 32-bit logits (no cap: a plain head)."""
+
+    def libraries(self):
+        return ["gemm", "elementwise"]
+
+    def forward(self, ctx, final):
+        logits = super().forward(ctx, final)
+        if self.spec.softcap is not None:
+            ctx.kernels.tanh_cap(logits, float(self.spec.softcap))
         return logits

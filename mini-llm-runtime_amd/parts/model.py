@@ -135,6 +135,8 @@ class DecoderModel:
         state theirs (the ends: `workspace_plan(rows, logits_rows, dtype, limits)`; blocks and their parts:
         `workspace_plan(rows, dtype, limits)`; a part without one gets its buffers on demand)."""
         plan = {("final", self.dtype): logits_rows * self.spec.hidden}
+        if any(run.add_embedding for run in self.spec.schedule):
+            plan[("embedding_copy", torch.float32)] = rows * self.spec.hidden
 
         def add(part_plan):
             for key, count in part_plan.items():
@@ -176,13 +178,33 @@ class DecoderModel:
         h = self.embed.forward(ctx)
         pending = None
         schedule = self.spec.schedule
+        again = None                 # the embedding's output, kept for the runs that add it to the stream again
+        if any(run.add_embedding for run in schedule):
+            again = ctx.workspace.get("embedding_copy", tuple(h.shape), torch.float32)
+            k.copy_float(h, again)
         for i, run in enumerate(schedule):
             # (the norm the next run starts with: a block may prepare it while it adds its last output into h)
             next_block = self.blocks[schedule[i + 1].layer] if i + 1 < len(schedule) else None
             next_norm = next_block.norm1 if next_block is not None else None
             block = self.blocks[run.layer]
             more = {"next_block": next_block} if getattr(block, "wants_next_block", False) else {}
+            # (the run after this one starts a further pass: the embedding's output joins the stream behind this run,
+            # by the block itself where it can take it into its last pass over the stream)
+            extra = again if i + 1 < len(schedule) and schedule[i + 1].add_embedding else None
+            if i == 0 and run.add_embedding:
+                raise PartError("the first run cannot add the embedding's output again")
+            if extra is not None and getattr(block, "adds_extra", False):
+                more["extra"], extra = extra, None
+            if extra is not None:
+                next_norm = None                          # (the stream is not complete when this block ends)
+                if "next_block" in more:
+                    more["next_block"] = None
             pending = block.forward(ctx, h, pending, self.cache_ids[run.cache], run.write_cache, next_norm=next_norm, **more)
+            if extra is not None:
+                if pending is not None and not isinstance(pending, Complete):
+                    k.residual_add(h, pending)
+                k.residual_add_float(h, extra)
+                pending = None
             if isinstance(pending, Complete) and i + 1 == len(schedule):
                 pending = None                            # (h is complete)
             if status is not None:                        # h + pending is the hidden state after this run

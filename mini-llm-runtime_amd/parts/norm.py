@@ -44,6 +44,45 @@ class RmsNorm:
         return out
 
 
+@register_part("norm", "tanh_norm")
+class TanhNorm:
+    """A norm that takes no mean and no variance: y = tanh(alpha x) * weight + bias, element by element, with one
+    learned number alpha a norm; 32-bit.  It serves in front of a sublayer (`forward`, on the residual stream) and
+    behind one (`add_into`: the norm of what the sublayer gave is added to the stream, and the norm in front of the
+    next sublayer may be taken in the same pass)."""
+    graph_safe = True
+
+    def __init__(self, spec):
+        self.size = spec.size
+        self.weight = self.bias = None
+        self.alpha = 1.0
+
+    def weight_specs(self):
+        return {"weight": WeightSpec((self.size,), keep_float32=True),
+                "bias": WeightSpec((self.size,), keep_float32=True, init=("normal", 0.0, 0.1)),
+                "alpha": WeightSpec((), keep_float32=True, init=("uniform", 0.3, 1.0))}
+
+    def bind(self, weights):
+        self.weight, self.bias = weights["weight"], weights["bias"]
+        self.alpha = float(weights["alpha"].detach().to("cpu", torch.float32).reshape(()))    # (one number, read once)
+
+    def libraries(self):
+        return ["elementwise"]
+
+    def params(self):
+        return self.weight, self.bias, self.alpha
+
+    def forward(self, ctx, h, delta, out, rows=None, write_h=True):
+        ctx.kernels.tanh_norm_rows(h, delta, self.weight, self.bias, self.alpha, out, rows=rows, write_h=write_h)
+        return out
+
+    def add_into(self, ctx, delta, h, extra=None, then=None, out=None):
+        """h += norm(delta) (+ extra, a float matrix like h); `then` (another norm of this kind) with `out`: out =
+        then(h) in the same pass."""
+        ctx.kernels.tanh_norm_add(delta, self.weight, self.bias, self.alpha, h, extra=extra,
+                                  then=then.params() if then is not None else None, out=out)
+
+
 @register_part("norm", "layernorm")
 class LayerNorm:
     """y = (x - mean) / sqrt(var + eps) * weight + bias, var the mean of the squared deviations; 32-bit."""

@@ -291,7 +291,11 @@ class DeltaRule:
     per head and key channel; per head S <- diag(g) S, u = beta (v - S^T k), S <- S + k u^T, o = S^T q.  Each head's o
     is divided by its root mean square over the value channels, multiplied by a weight the heads share and by
     sigmoid(Wg2 (Wg1 x)), and projected by Wo.  A request's state is S [heads, head_dim, value_dim] and the
-    convolution's last taps - 1 inputs.  Decays, beta, the unit norms and the state are 32-bit."""
+    convolution's last taps - 1 inputs.  Decays, beta, the unit norms and the state are 32-bit.
+
+    `decay` "head": ONE decay for all key channels of a head, g = exp(-exp(A_log) softplus(Wa x + dt_bias)) with Wa
+    [heads, hidden] (tensor `a`) instead of the low-rank pair.  `gate` "silu": the read-out's gate is silu(Wg x) with a
+    full matrix Wg (tensor `g`, which then rides behind q, k, v in the one projection) instead of the low-rank sigmoid."""
     graph_safe = True
 
     def __init__(self, spec):
@@ -302,8 +306,13 @@ class DeltaRule:
             raise PartError(f"head_dim {s.head_dim}: the recurrence kernel takes up to 256 key channels a head")
         if not 1 <= s.conv_taps <= 8:
             raise PartError(f"conv_taps {s.conv_taps}: the convolution kernel takes 1 to 8 taps")
+        self.head_decay = getattr(s, "decay", "channel_low_rank") == "head"
+        self.full_gate = getattr(s, "gate", "low_rank_sigmoid") == "silu"
+        if getattr(s, "decay", "channel_low_rank") not in ("channel_low_rank", "head") or \
+                getattr(s, "gate", "low_rank_sigmoid") not in ("low_rank_sigmoid", "silu"):
+            raise PartError("delta rule: decay is channel_low_rank or head, gate is low_rank_sigmoid or silu")
         self.qk_width, self.v_width = s.kv_heads * s.head_dim, s.heads * s.value_dim
-        self.decay_width = s.heads * s.head_dim
+        self.decay_width = s.heads if self.head_decay else s.heads * s.head_dim
         self.channels = 2 * self.qk_width + self.v_width
         self.state_floats = s.heads * s.head_dim * s.value_dim
         self.out_name = "mixer_out"
@@ -314,25 +323,44 @@ class DeltaRule:
     def weight_specs(self):
         s = self.spec
         taps = lambda n: WeightSpec((n, s.conv_taps), keep_float32=True, init=("normal", 0.0, 0.4))
-        return {"q": WeightSpec((self.qk_width, s.hidden), stack="in"), "k": WeightSpec((self.qk_width, s.hidden), stack="in"),
-                "v": WeightSpec((self.v_width, s.hidden), stack="in"),
-                "a1": WeightSpec((s.decay_rank, s.hidden)), "g1": WeightSpec((s.gate_rank, s.hidden)),
-                "b": WeightSpec((s.heads, s.hidden)),
-                "q.conv": taps(self.qk_width), "k.conv": taps(self.qk_width), "v.conv": taps(self.v_width),
-                "a2": WeightSpec((self.decay_width, s.decay_rank), init=("normal", 0.0, 0.3)),
-                "dt_bias": WeightSpec((self.decay_width,), keep_float32=True, init=("uniform", -4.0, 0.0)),
-                "A_log": WeightSpec((s.heads,), keep_float32=True, init=("uniform", -1.0, 1.5)),
-                "g2": WeightSpec((self.v_width, s.gate_rank), init=("normal", 0.0, 0.3)),
-                "norm": WeightSpec((s.value_dim,), keep_float32=True), "o": WeightSpec((s.hidden, self.v_width))}
+        specs = {"q": WeightSpec((self.qk_width, s.hidden), stack="in"), "k": WeightSpec((self.qk_width, s.hidden), stack="in"),
+                 "v": WeightSpec((self.v_width, s.hidden), stack="in")}
+        if self.full_gate:
+            specs["g"] = WeightSpec((self.v_width, s.hidden), stack="in")
+        else:
+            specs.update({"g1": WeightSpec((s.gate_rank, s.hidden)),
+                          "g2": WeightSpec((self.v_width, s.gate_rank), init=("normal", 0.0, 0.3))})
+        if self.head_decay:
+            specs["a"] = WeightSpec((s.heads, s.hidden))
+        else:
+            specs.update({"a1": WeightSpec((s.decay_rank, s.hidden)),
+                          "a2": WeightSpec((self.decay_width, s.decay_rank), init=("normal", 0.0, 0.3))})
+        specs.update({"b": WeightSpec((s.heads, s.hidden)),
+                      "q.conv": taps(self.qk_width), "k.conv": taps(self.qk_width), "v.conv": taps(self.v_width),
+                      "dt_bias": WeightSpec((self.decay_width,), keep_float32=True, init=("uniform", -4.0, 0.0)),
+                      "A_log": WeightSpec((s.heads,), keep_float32=True, init=("uniform", -1.0, 1.5)),
+                      "norm": WeightSpec((s.value_dim,), keep_float32=True), "o": WeightSpec((s.hidden, self.v_width))})
+        return specs
 
     def bind(self, weights):
-        self.proj = stacked([weights[n] for n in ("q", "k", "v")])
+        self.proj = stacked([weights[n] for n in ("q", "k", "v") + (("g",) if self.full_gate else ())])
         self.conv = torch.cat([weights["q.conv"], weights["k.conv"], weights["v.conv"]]).contiguous()
-        self.a1, self.g1, self.beta = weights["a1"], weights["g1"], weights["b"]
-        self.a2, self.g2 = weights["a2"], weights["g2"]
-        self.decay_rank, self.gate_rank = self.a1.shape[0], self.g1.shape[0]
-        if self.a2.shape[1] != self.decay_rank or self.g2.shape[1] != self.gate_rank:
-            raise PartError("the low-rank pairs of the decay or of the gate do not fit each other")
+        self.beta = weights["b"]
+        if self.head_decay:
+            self.a1, self.a2, self.decay_rank = weights["a"], None, 0
+        else:
+            self.a1, self.a2 = weights["a1"], weights["a2"]
+            self.decay_rank = self.a1.shape[0]
+            if self.a2.shape[1] != self.decay_rank:
+                raise PartError("the low-rank pair of the decay does not fit itself")
+        if self.full_gate:
+            self.g1 = self.g2 = None
+            self.gate_rank = 0
+        else:
+            self.g1, self.g2 = weights["g1"], weights["g2"]
+            self.gate_rank = self.g1.shape[0]
+            if self.g2.shape[1] != self.gate_rank:
+                raise PartError("the low-rank pair of the gate does not fit itself")
         self.dt_bias, self.a_log, self.norm, self.o = weights["dt_bias"], weights["A_log"], weights["norm"], weights["o"]
 
     def cache_spec(self):
@@ -343,7 +371,8 @@ class DeltaRule:
 
     def workspace_plan(self, rows, dtype, limits):
         s = self.spec
-        return {("delta_proj", dtype): rows * self.channels, ("delta_conv", dtype): rows * self.channels,
+        return {("delta_proj", dtype): rows * (self.channels + (self.v_width if self.full_gate else 0)),
+                ("delta_conv", dtype): rows * self.channels,
                 ("delta_low_a", dtype): rows * self.decay_rank, ("delta_low_g", dtype): rows * self.gate_rank,
                 ("delta_z", torch.float32): rows * self.decay_width,
                 ("log_decay", torch.float32): rows * self.decay_width, ("delta_beta", torch.float32): rows * s.heads,
@@ -372,26 +401,33 @@ class DeltaRule:
         k.gemm(x, self.proj, proj)
         live, stage = ctx.cache.state_view(cache_id), ctx.cache.state_stage(cache_id)
         conv = ws.get("delta_conv", (m, self.channels), x.dtype)
-        k.causal_conv(proj, self.conv, None, conv, live, stage, self.state_floats, ctx.slots, ctx.positions,
+        k.causal_conv(proj[:, :self.channels], self.conv, None, conv, live, stage, self.state_floats, ctx.slots, ctx.positions,
                       silu=True, write_state=write_cache)
-        # the decays: a low-rank pair whose second product leaves 32-bit sums, then softplus and the head's rate
-        low_a = ws.get("delta_low_a", (m, self.decay_rank), x.dtype)
-        k.gemm(x, self.a1, low_a)
+        # the decays: 32-bit sums of a projection (one a head, or a low-rank pair's second product a key channel), then
+        # softplus and the head's rate
         z = ws.get("delta_z", (m, self.decay_width), torch.float32)
-        k.gemm(low_a, self.a2, z)
+        if self.head_decay:
+            k.gemm(x, self.a1, z)
+        else:
+            low_a = ws.get("delta_low_a", (m, self.decay_rank), x.dtype)
+            k.gemm(x, self.a1, low_a)
+            k.gemm(low_a, self.a2, z)
         log_decay = ws.get("log_decay", (m, self.decay_width), torch.float32)
-        k.channel_log_decay(z, self.dt_bias, self.a_log, log_decay, s.heads, s.head_dim)
-        low_g = ws.get("delta_low_g", (m, self.gate_rank), x.dtype)
-        k.gemm(x, self.g1, low_g)
-        gate = ws.get("delta_gate", (m, self.v_width), x.dtype)
-        k.gemm(low_g, self.g2, gate)
+        k.channel_log_decay(z, self.dt_bias, self.a_log, log_decay, s.heads, 1 if self.head_decay else s.head_dim)
+        if self.full_gate:
+            gate = proj[:, self.channels:]
+        else:
+            low_g = ws.get("delta_low_g", (m, self.gate_rank), x.dtype)
+            k.gemm(x, self.g1, low_g)
+            gate = ws.get("delta_gate", (m, self.v_width), x.dtype)
+            k.gemm(low_g, self.g2, gate)
         beta = ws.get("delta_beta", (m, s.heads), torch.float32)       # (the sigmoid is the recurrence kernel's)
         k.gemm(x, self.beta, beta)
         first, count, n = _requests(ctx)
         a, b = self.qk_width, 2 * self.qk_width
         o = ws.get("recurrent_out", (m, self.v_width), torch.float32)
         more = dict(heads_per_group=s.heads // s.kv_heads, q_scale=float(s.head_dim) ** -0.5, unit_eps=float(s.unit_eps),
-                    write_state=write_cache)
+                    write_state=write_cache, decay_per_head=self.head_decay)
         chunks_most = m // DELTA_CHUNK + len(ctx.segments)
         if ctx.dtype == torch.bfloat16 and m >= max(CHUNKS_FROM, 8 * len(ctx.segments)) and s.head_dim <= k.DELTA_CHUNK_MAX_KEYS and \
                 k.delta_chunk_floats(chunks_most, s.heads, s.head_dim, s.value_dim) <= PIECE_FLOATS:
@@ -405,7 +441,8 @@ class DeltaRule:
             k.delta_rule(conv[:, :a], conv[:, a:b], conv[:, b:], log_decay, beta, o, live, stage, 0, first, count, n, ctx.slots,
                          s.heads, s.head_dim, s.value_dim, **more)
         y = ws.get("recurrent_normed", (m, self.v_width), x.dtype)
-        k.gated_part_norm(o, gate, self.norm, y, s.value_dim, float(s.eps), gate_first=False, gate_kind="sigmoid")
+        k.gated_part_norm(o, gate, self.norm, y, s.value_dim, float(s.eps), gate_first=False,
+                          gate_kind="silu" if self.full_gate else "sigmoid")
         out = ws.get(self.out_name, (m, s.hidden), x.dtype)
         k.gemm(y, self.o, out)
         return out

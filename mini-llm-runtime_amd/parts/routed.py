@@ -1,7 +1,9 @@
 """A mixture of experts with group-limited routing.  Every token scores all experts, s = sigmoid(router . x) in
 32-bit (an ordinary product with float output); the experts form equal groups of neighbours, a group's score is the sum of its two largest s, and only
 experts of the best groups can be chosen; of those the `top` largest s win and weigh their experts' outputs (as
-they are, or divided by their sum).  An expert is an ungated feed-forward down(act(up(x))).
+they are, or divided by their sum, and times `route_scale`).  With `correction` the choice goes by s plus a stored
+number an expert while the weights stay the plain s.  An expert is an ungated feed-forward down(act(up(x))) or,
+`gated`, down(act(gate(x)) * up(x)).
 
 The step's (token, expert) pairs are sorted by expert on the device, so that every expert's rows lie side by side
 and ONE launch multiplies all of them with their own weights (`Kernels.experts_gemm`, the rows of the first product
@@ -21,10 +23,15 @@ class RoutedMlp:
 
     def __init__(self, spec):
         s = self.spec = spec
-        if s.activation not in ACTIVATIONS:
+        self.gated = bool(getattr(s, "gated", False))
+        if self.gated:
+            if s.activation not in ("silu", "gelu_tanh"):
+                raise PartError(f"gated experts: activation {s.activation!r} is not built (silu, gelu_tanh)")
+        elif s.activation not in ACTIVATIONS:
             raise PartError(f"activation {s.activation!r} is not built ({', '.join(ACTIVATIONS)})")
-        if s.score != "sigmoid" or s.renormalize:
-            raise PartError("routing: sigmoid scores used as they are is what is built")
+        if s.score != "sigmoid":
+            raise PartError("routing: sigmoid scores are what is built")
+        self.correction = None
         if s.experts % s.group_count != 0 or not 1 <= s.group_keep <= s.group_count or \
                 not 1 <= s.top <= s.group_keep * (s.experts // s.group_count):
             raise PartError(f"routing: {s.experts} experts in {s.group_count} groups of which {s.group_keep} stay cannot "
@@ -36,7 +43,11 @@ class RoutedMlp:
         # (a matrix like the others: its products with the layer's input are exact in 32 bits, and so are their sums'
         # partial results up to rounding: the logits are an ordinary product with float output)
         specs = {"router": WeightSpec((s.experts, s.hidden), init=("normal", 0.0, 0.05))}
+        if getattr(s, "correction", False):
+            specs["correction"] = WeightSpec((s.experts,), keep_float32=True, init=("normal", 0.0, 0.05))
         for e in range(s.experts):
+            if self.gated:                      # (an expert's gate and up side by side: one product gives both)
+                specs[f"e{e}.gate"] = WeightSpec((s.intermediate, s.hidden), stack="up")
             specs[f"e{e}.up"] = WeightSpec((s.intermediate, s.hidden), stack="up")
         for e in range(s.experts):
             specs[f"e{e}.down"] = WeightSpec((s.hidden, s.intermediate), stack="down")
@@ -45,11 +56,13 @@ class RoutedMlp:
     def bind(self, weights):
         s = self.spec
         self.router = weights["router"]
-        self.up = stacked([weights[f"e{e}.up"] for e in range(s.experts)]).view(s.experts, s.intermediate, s.hidden)
+        self.correction = weights.get("correction")
+        first = [weights[f"e{e}.{n}"] for e in range(s.experts) for n in (("gate", "up") if self.gated else ("up",))]
+        self.up = stacked(first).view(s.experts, (2 if self.gated else 1) * s.intermediate, s.hidden)
         self.down = stacked([weights[f"e{e}.down"] for e in range(s.experts)]).view(s.experts, s.hidden, s.intermediate)
 
     def libraries(self):
-        return ["gemm", "grouped_gemm"]
+        return ["gemm", "grouped_gemm"] + (["elementwise"] if self.gated else [])
 
     def workspace_plan(self, rows, dtype, limits):
         s = self.spec
@@ -58,6 +71,7 @@ class RoutedMlp:
                 ("route_weights", torch.float32): pairs,
                 ("route_offsets", torch.int32): s.experts + 1, ("route_token", torch.int32): pairs,
                 ("route_row", torch.int32): pairs, ("route_act", dtype): pairs * s.intermediate,
+                **({("route_gate_up", dtype): pairs * 2 * s.intermediate} if self.gated else {}),
                 ("route_y", dtype): pairs * s.hidden, ("ffn_out", dtype): rows * s.hidden}
 
     def forward(self, ctx, x):
@@ -72,10 +86,16 @@ class RoutedMlp:
         row_of = ws.get("route_row", (pairs,), torch.int32)
         logits = ws.get("route_logits", (m, s.experts), torch.float32)
         k.gemm(x, self.router, logits)                   # 32-bit sums of the engine's element type's products
-        k.router_topk(logits, ids, weights, s.group_count, s.group_keep)
+        k.router_topk(logits, ids, weights, s.group_count, s.group_keep, correction=self.correction,
+                      renormalize=bool(s.renormalize), scale=float(getattr(s, "route_scale", 1.0)))
         k.route_sort(ids, s.experts, offsets, token_of, row_of)
         act = ws.get("route_act", (pairs, s.intermediate), x.dtype)
-        k.experts_gemm(x, self.up, act, offsets, gather=token_of, act=s.activation)
+        if self.gated:
+            both = ws.get("route_gate_up", (pairs, 2 * s.intermediate), x.dtype)
+            k.experts_gemm(x, self.up, both, offsets, gather=token_of)
+            k.gated_act_mul(both, act, s.activation)
+        else:
+            k.experts_gemm(x, self.up, act, offsets, gather=token_of, act=s.activation)
         y = ws.get("route_y", (pairs, s.hidden), x.dtype)
         k.experts_gemm(act, self.down, y, offsets)
         out = ws.get("ffn_out", (m, s.hidden), x.dtype)

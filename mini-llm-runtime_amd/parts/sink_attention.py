@@ -15,7 +15,8 @@ rotated key part that all heads share; only the latent vector and that part are 
 The up-projections are moved to the query's side: q_lat[h] = W_uk[h]^T q_plain[h], so a head's score is
 q_lat[h] . latent + q_rot[h] . k_rot -- attention of all heads over ONE shared key row whose first `rank` channels
 are also the value -- and the head's output is W_uv[h] applied to the attention's latent result.  With `q_rank` the
-queries come through a normed latent of their own, q = W_uq norm(W_dq x).
+queries come through a normed latent of their own, q = W_uq norm(W_dq x).  With `head_gate` every head's output is
+multiplied by ONE number, sigmoid(Wg x)[head], before the output projection.
 """
 from __future__ import annotations
 
@@ -200,7 +201,10 @@ class LatentAttention:
         self.row = s.rank + s.rot_dim                    # a token's cache row, and a query head after the move
         self.o_width = s.heads * s.value_dim
         self.out_name = "mixer_out"
-        self.proj = self.o = self.norm = self.uk_t = self.uv = self.sink = self.uq = self.q_norm = None
+        self.head_gate = getattr(s, "head_gate", None)
+        if self.head_gate not in (None, "sigmoid"):
+            raise PartError(f"head_gate {self.head_gate!r}: sigmoid or none")
+        self.proj = self.o = self.norm = self.uk_t = self.uv = self.sink = self.uq = self.q_norm = self.gate = None
 
     def weight_specs(self):
         s = self.spec
@@ -215,14 +219,17 @@ class LatentAttention:
                  "o": WeightSpec((s.hidden, self.o_width))}
         if s.sink:
             specs["sink"] = WeightSpec((s.heads,), keep_float32=True, init=("normal", 0.0, 1.0))
+        if self.head_gate is not None:      # (with a query latent it rides behind the two latents in the one projection)
+            specs["g"] = WeightSpec((s.heads, s.hidden), stack="down" if s.q_rank is not None else None)
         return specs
 
     def bind(self, weights):
         s = self.spec
         if s.q_rank is None:
             self.proj = stacked([weights["q"], weights["dkv"]])
+            self.gate = weights["g"] if self.head_gate is not None else None
         else:
-            self.proj = stacked([weights["dq"], weights["dkv"]])
+            self.proj = stacked([weights["dq"], weights["dkv"]] + ([weights["g"]] if self.head_gate is not None else []))
             self.uq, self.q_norm = weights["uq"], weights["dq.norm"]
         self.norm = weights["dkv.norm"]
         # the key up-projection as the queries meet it: per head [rank, head_dim]
@@ -241,7 +248,10 @@ class LatentAttention:
         s = self.spec
         first = self.q_width if s.q_rank is None else s.q_rank
         more = {} if s.q_rank is None else {("latent_cq", dtype): rows * s.q_rank, ("latent_queries", dtype): rows * self.q_width}
-        return {("latent_proj", dtype): rows * (first + self.row), ("latent_q", dtype): rows * s.heads * self.row,
+        if self.head_gate is not None:
+            more[("latent_gate", dtype)] = rows * s.heads
+        return {("latent_proj", dtype): rows * (first + self.row + (s.heads if self.head_gate is not None else 0)),
+                ("latent_q", dtype): rows * s.heads * self.row,
                 ("latent_out", dtype): rows * s.heads * s.rank, ("attn", dtype): rows * self.o_width,
                 (self.out_name, dtype): rows * s.hidden, **more, **_groups_plan(rows, s.heads, 1, s.rank)}
 
@@ -256,8 +266,12 @@ class LatentAttention:
         pages = view.tensors["latent"]
         q = ctx.workspace.get("latent_q", (m, s.heads * self.row), x.dtype)
         rope, interleaved = _rope_table(self.position, ctx, x.device, s.rot_dim)
+        gate = None
         if s.q_rank is None:
             queries, q_ld = proj, ld
+            if self.head_gate is not None:
+                gate = ctx.workspace.get("latent_gate", (m, s.heads), x.dtype)
+                k.gemm(x, self.gate, gate)
             k.latent_prep(proj, q, pages, view.block_table, ctx.slots, ctx.positions, self.norm, float(s.eps), rope, s.heads,
                           s.head_dim, s.rot_dim, s.rank, view.page_size, write_cache, interleaved=interleaved)
         else:
@@ -266,7 +280,9 @@ class LatentAttention:
             k.rmsnorm_columns(proj[:, :s.q_rank], self.q_norm, cq, float(s.eps))
             queries, q_ld = ctx.workspace.get("latent_queries", (m, self.q_width), x.dtype), self.q_width
             k.gemm(cq, self.uq, queries)
-            k.latent_prep(proj[:, s.q_rank:], q, pages, view.block_table, ctx.slots, ctx.positions, self.norm, float(s.eps),
+            if self.head_gate is not None:
+                gate = proj[:, s.q_rank + self.row:]
+            k.latent_prep(proj[:, s.q_rank:s.q_rank + self.row], q, pages, view.block_table, ctx.slots, ctx.positions, self.norm, float(s.eps),
                           rope, s.heads, s.head_dim, s.rot_dim, s.rank, view.page_size, write_cache, q_src=queries,
                           interleaved=interleaved)
         # the plain query channels through the key up-projection, head by head, into the first `rank` channels
@@ -277,6 +293,8 @@ class LatentAttention:
                self.mask_size)
         attn = ctx.workspace.get("attn", (m, self.o_width), x.dtype)
         k.heads_gemm(lat.view(m, s.heads, s.rank), self.uv, attn.view(m, s.heads, s.value_dim))
+        if gate is not None:
+            k.head_gate_mul(attn, gate, attn, s.heads)
         out = ctx.workspace.get(self.out_name, (m, s.hidden), x.dtype)
         k.gemm(attn, self.o, out)
         return out
