@@ -119,4 +119,4 @@ def write_safetensors(path, tensors, metadata=None):
         f.write(text)
         for t in ordered:                                  # (straight from the tensor's memory: no second copy)
             if t.numel():
-                f.write(memoryview(t.view(torch.uint8).reshape(-1).numpy()))
+                f.write(memoryview(t.reshape(-1).view(torch.uint8).numpy()))      # (reshape first: a scalar has no axis to widen)

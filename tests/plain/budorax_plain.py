@@ -120,7 +120,7 @@ def short_convolution(x, taps):
     """x [T, C], taps [C, n]: y_t = sum_j taps[:, n - 1 - j] x_(t - j), zeros before the sequence."""
     T, n = x.shape[0], taps.shape[1]
     y = np.zeros_like(x)
-    for j in range(n):
+    for j in range(min(n, T)):
         y[j:] += x[:T - j] * taps[:, n - 1 - j]
     return y
 
@@ -167,11 +167,16 @@ def choose_experts(x, w, router):
     return ids, picked / (picked.sum(axis=-1, keepdims=True) + 1e-20) * router["scale"]
 
 
-def choice_margin(x, w, router):
-    """Per token, the gap between the last chosen and the first left-out choice score (inf when all are chosen)."""
-    choice = np.sort(sigmoid(x @ w["router"].T) + w["correction"], axis=-1)[:, ::-1]
+def choice_margin(x, w, router, rounding=2.0 ** -8):
+    """[T]: the gap between the last chosen and the first left-out choice score (infinite when all are chosen), in units
+    of how far rounding every element of x by `rounding` (relative) may move a score.  A comparison with an engine that
+    rounds may not rest on tokens whose margin is a small number."""
+    s = sigmoid(x @ w["router"].T)
+    moved = (s * (1.0 - s) * rounding * np.sqrt((x * x) @ (w["router"] ** 2).T)).max(axis=1) + 1e-300
+    choice = -np.sort(-(s + w["correction"]), axis=-1)
     top = router["top"]
-    return choice[:, top - 1] - choice[:, top] if top < choice.shape[1] else np.full(x.shape[0], np.inf)
+    gap = choice[:, top - 1] - choice[:, top] if top < choice.shape[1] else np.full(x.shape[0], np.inf)
+    return gap / moved
 
 
 def expert(x, w, e):
@@ -181,9 +186,10 @@ def expert(x, w, e):
 def expert_mixture(x, w, cfg):
     ids, weights = choose_experts(x, w, cfg["router"])
     out = np.zeros_like(x)
-    for t in range(x.shape[0]):
-        for e, a in zip(ids[t], weights[t]):
-            out[t] += a * expert(x[t:t + 1], w, int(e))[0]
+    for e in range(cfg["router"]["experts"]):
+        rows, which = np.nonzero(ids == e)
+        if len(rows):
+            out[rows] += weights[rows, which][:, None] * expert(x[rows], w, e)
     return out
 
 
@@ -235,3 +241,55 @@ def forward(config, weights, tokens, streams=None, margins=None):
     logits = named_norm(weights, "final.norm", x) @ table.T
     cap = config["logit_softcap"]
     return cap * np.tanh(logits / cap)
+
+
+class PlainBudorax:
+    """A model folder (config.json, model.safetensors) run by the functions above."""
+
+    def __init__(self, folder):
+        import json
+        import os
+
+        import torch
+        from safetensors.torch import load_file
+        with open(os.path.join(folder, "config.json")) as f:
+            self.cfg = json.load(f)
+        self.tensors = {n: (t.to(torch.float64) if t.dtype.is_floating_point else t).numpy()
+                        for n, t in load_file(os.path.join(folder, "model.safetensors")).items()}
+
+    def logits(self, tokens, want=None):
+        rows = forward(self.cfg, self.tensors, tokens)
+        return rows if want is None else rows[np.asarray(want, dtype=np.int64)]
+
+    def streams(self, tokens):
+        out = []
+        forward(self.cfg, self.tensors, tokens, streams=out)
+        return np.stack(out)
+
+    def routing_margins(self, tokens):
+        """[T]: every token's smallest choice margin over the layer runs, or None for a model without experts."""
+        margins = []
+        forward(self.cfg, self.tensors, tokens, margins=margins)
+        return np.min(margins, axis=0) if margins else None
+
+    def decisive(self, tokens, rng, least=40.0, tries=2000):
+        """`tokens` with the token at every position whose routing is a close call (a margin below `least`) drawn
+        again, from left to right (a position's margins depend on the tokens up to it only), so that an engine that
+        rounds chooses the experts this file chooses."""
+        tokens = list(tokens)
+        vocab = self.tensors["embed"].shape[0]
+        for _ in range(tries):
+            margins = self.routing_margins(tokens)
+            near = [] if margins is None else np.nonzero(margins < least)[0]
+            if len(near) == 0:
+                return tokens
+            tokens[int(near[0])] = int(rng.integers(0, vocab))
+        raise ValueError("no decisive sequence found")
+
+    def greedy(self, prompt, n):
+        tokens, out = list(prompt), []
+        for _ in range(n):
+            t = int(np.argmax(self.logits(tokens, [len(tokens) - 1])[0]))
+            out.append(t)
+            tokens.append(t)
+        return out
