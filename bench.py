@@ -26,6 +26,9 @@ many gigabytes).  Every runner is built with the product's own defaults.  One JS
     chunked grouped-query attention beside a mixture of experts, in turn).
   * --only tigelorn: the same for Tigelorn models (windowed attention beside constant-decay linear attention, the
     gated delta rule, latent attention with a query latent, in turn), beside a Taletar model of equal sizes.
+  * --only budorax: the same for Budorax models (differential attention in blocks of positions, latent attention with a
+    gate a head, the gated delta rule with a decay a head, each between two norms and beside a mixture of gated experts;
+    two of the six layers run twice), beside a Tigelorn model of equal sizes.
 """
 import argparse
 import json
@@ -637,6 +640,97 @@ class TigelornBench(Bench):
                     frac=round(step_bytes / (seconds / steps) / HBM_PEAK, 5)), step_bytes, report
 
 
+# `--only budorax`: layer sizes that resemble a real model's, for a Budorax model of six layers -- differential attention
+# in blocks of positions, latent attention with a query latent and a gate a head, the gated delta rule with one decay a
+# head, differential attention, latent attention, the delta rule -- of which the third and the fourth run twice (eight
+# runs a token), every layer beside a mixture of eight gated experts of which a token uses two (an expert has half the
+# dense inner size: a token's feed-forward work equals the dense one's), and for the closest model the engine had
+# before: a Tigelorn model (eight layers: the delta rule, latent attention with a query latent, windowed attention
+# beside linear attention) of the same width, feed-forward and heads.
+BUDORAX_SIZES = {
+    "2k": dict(width=2048, ff=5632, vocab=32000, layers=8, heads=16, kv_heads=4, chunk=1024, kv_rank=512, q_rank=768),
+    "4k": dict(width=4096, ff=12288, vocab=32000, layers=8, heads=32, kv_heads=8, chunk=1024, kv_rank=512, q_rank=1536),
+}
+
+
+class BudoraxBench(Bench):
+    """A Budorax model of BUDORAX_SIZES[size] with random weights drawn on the GPU."""
+    EXPERTS, TOP = 8, 2
+
+    def __init__(self, size, args):
+        import torch
+        from mini_llm_runtime_amd.api import parse_dtype
+        from mini_llm_runtime_amd.config import config_from_dict
+        from mini_llm_runtime_amd.parts import DecoderModel, expected_tensors
+        from mini_llm_runtime_amd.weights import random_tensors_on_device
+        d = BUDORAX_SIZES[size]
+        self.torch, self.args, self.size = torch, args, size
+        self.dtype = parse_dtype(args.dtype)
+        self.tag = "bf16" if self.dtype == torch.bfloat16 else "fp32"
+        h = d["heads"]
+        mlp = dict(kind="moe", expert=dict(ff=d["ff"] // 2), router=dict(experts=self.EXPERTS, top=self.TOP, scale=1.5))
+        # (two maps of 64 channels a head: the query/key work of one 128-channel head)
+        attention = dict(type="attention", mlp=mlp,
+                         mixer=dict(heads=h, kv_heads=d["kv_heads"], dim=64, vdim=128, diff=0.6, scale=64 ** -0.5,
+                                    rot=dict(dims=64, base=1000000.0), mask=dict(size=d["chunk"])))
+        latent = dict(type="latent_attention", mlp=mlp,
+                      mixer=dict(heads=h, dim=128, rot_dim=64, vdim=128, kv_rank=d["kv_rank"], q_rank=d["q_rank"], scale=192 ** -0.5,
+                                 rot=dict(dims=64, base=10000.0)))
+        delta = dict(type="delta", mlp=mlp, mixer=dict(heads=h, kv_heads=h // 2, dim=128, vdim=128, conv=4))
+        layers = [attention, latent, delta, attention, latent, delta]
+        self.cfg = config_from_dict(dict(architecture="Budorax", vocab=d["vocab"], width=d["width"], norm=dict(eps=1e-5),
+                                         logit_softcap=30.0, loop=dict(start=2, stop=4, times=2), layers=layers))
+        self.model = DecoderModel(self.cfg, random_tensors_on_device(expected_tensors(self.cfg), 0, self.dtype, "cuda"),
+                                  self.dtype, "cuda:0")
+        self.layers = self.full_layers = len(self.model.spec.schedule)
+        self.weights_from = "drawn on the GPU"
+        self.elem = 2 if self.dtype == torch.bfloat16 else 4
+        w = d["width"]
+        expert = 3 * w * (d["ff"] // 2)                           # elements of one expert
+        runs = [run.layer for run in self.model.spec.schedule]
+        kinds = [layers[i]["type"] for i in runs]
+        # elements of a layer without its experts: what every token multiplies with
+        def shared(i):
+            total = 0
+            for part in self.model.blocks[i].parts().values():
+                total += sum(v.numel() for v in vars(part).values() if isinstance(v, torch.Tensor) and v.dim() >= 2)
+            return total - self.EXPERTS * expert
+        self.shared = [shared(i) for i in range(len(layers))]
+        self.expert = expert
+        self.runs = runs
+        self.matrix_params = sum(self.shared[i] + self.TOP * expert for i in runs)
+        self.weight_bytes = self.model.weight_bytes()             # (the table once, as the head)
+        n_attention, n_latent, n_delta = (kinds.count(t) for t in ("attention", "latent_attention", "delta"))
+        # cache rows that a decoding token's attention reads: both maps' keys and the values of the kv heads over its
+        # block, the latent row once for all heads over the whole context; recurrent state read and written a step
+        self.block_row_bytes = n_attention * d["kv_heads"] * (2 * 64 + 128) * self.elem
+        self.latent_row_bytes = n_latent * (d["kv_rank"] + 64) * self.elem
+        self.state_bytes = n_delta * h * 128 * 128 * 4 * 2
+        self.kv_bytes_per_token = 0                  # (see decode_point)
+        seen = lambda t: sum(p % d["chunk"] + 1 for p in range(t))
+        self.attention_flops = lambda t: (n_attention * 2.0 * seen(t) * h * (2 * 64 + 2 * 128)
+                                          + n_latent * 2.0 * (t * (t + 1) / 2) * h * (2 * d["kv_rank"] + 64)
+                                          + n_delta * 3 * 2.0 * t * h * 128 * 128)
+        self.vocab = d["vocab"]
+        self.g = torch.Generator().manual_seed(0)
+
+    def prefill_flops(self, t):
+        d = BUDORAX_SIZES[self.size]
+        return 2.0 * t * self.matrix_params + self.attention_flops(t) + 2.0 * d["vocab"] * d["width"]
+
+    def decode_point(self, batch, steps, warmup, context=None):
+        d = BUDORAX_SIZES[self.size]
+        seconds, mean_context, report = self.decode(batch, steps, warmup, context)
+        # weights a step reads: a layer's shared matrices and the experts its tokens choose (about E (1 - (1 - top / E)^batch)
+        # of them), once for every run of the layer; the table as the head
+        touched = self.EXPERTS * (1.0 - (1.0 - self.TOP / self.EXPERTS) ** batch)
+        weights = (sum(self.shared[i] + touched * self.expert for i in self.runs) + d["vocab"] * d["width"]) * self.elem
+        step_bytes = weights + batch * ((mean_context % d["chunk"] + 1) * self.block_row_bytes
+                                        + mean_context * self.latent_row_bytes + self.state_bytes)
+        return dict(tok_s=round(batch * steps / seconds, 1), ms=round(seconds / steps * 1e3, 4),
+                    frac=round(step_bytes / (seconds / steps) / HBM_PEAK, 5)), step_bytes, report
+
+
 def design_block(args):
     """Prefill (2048 tokens in one step) and decode (batch 8 and 64 behind --context tokens) of a design's sizes
     beside the closest model the engine had before it (a Qwen3 dense model of equal width, heads, feed-forward and
@@ -645,8 +739,8 @@ def design_block(args):
     import copy
     out = {}
     design = getattr(args, "design", "taletar")
-    table, make_design = {"pamunex": (PAMUNEX_SIZES, PamunexBench), "tigelorn": (TIGELORN_SIZES, TigelornBench)}.get(
-        design, (DESIGN_SIZES, TaletarBench))
+    table, make_design = {"pamunex": (PAMUNEX_SIZES, PamunexBench), "tigelorn": (TIGELORN_SIZES, TigelornBench),
+                          "budorax": (BUDORAX_SIZES, BudoraxBench)}.get(design, (DESIGN_SIZES, TaletarBench))
     for size in (args.design_sizes.split(",") if args.design_sizes else list(table)):
         d = table[size]
         dense = (d["layers"], dict(hidden_size=d["width"], num_attention_heads=d["heads"], num_key_value_heads=d["kv_heads"],
@@ -655,6 +749,7 @@ def design_block(args):
                                    tie_word_embeddings=False))
         block = {}
         beside = ("taletar", lambda a: TaletarBench(size, a)) if design == "tigelorn" else \
+            ("tigelorn", lambda a: TigelornBench(size, a)) if design == "budorax" else \
             ("qwen3_dense", lambda a: Bench(size, 0, a, sizes=dense))
         for name, make in ((design, lambda a: make_design(size, a)), beside):
             plain_args, profiled = copy.copy(args), copy.copy(args)
@@ -697,12 +792,12 @@ def main():
                          "tensors drawn on the GPU; auto: folder for the 0.6B sizes, gpu for the larger ones")
     ap.add_argument("--warm-up", type=int, default=0,
                     help="--only engine: 1 captures the decoding steps (Engine.warm_up) before the first burst")
-    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "prompt", "engine", "mixed", "taletar", "pamunex", "tigelorn"],
+    ap.add_argument("--only", default="all", choices=["all", "decode", "prefill", "prompt", "engine", "mixed", "taletar", "pamunex", "tigelorn", "budorax"],
                     help="profiling aid: run just the decode steps, just the prefill or just the mixed step; prompt: one "
                          "prompt of --context tokens in portions of 2048; engine: the "
                          "scheduler over a burst of requests (3 x batch requests of 512 prompt and 128 output tokens, "
                          "batch slots), printed as one line of its own")
-    ap.add_argument("--design-sizes", default="", help="--only taletar / pamunex / tigelorn: which of its sizes (2k, 4k; default both)")
+    ap.add_argument("--design-sizes", default="", help="--only taletar / pamunex / tigelorn / budorax: which of its sizes (2k, 4k; default both)")
     ap.add_argument("--library", type=int, default=1,
                     help="0: every matrix product on the hand-written kernels, none in the vendor library")
     ap.add_argument("--split-keys", type=int, default=256, help="the smallest range of keys of one attention workgroup")
@@ -726,7 +821,7 @@ def main():
     if not args.tune:
         from mini_llm_runtime_amd.kernels import build
         build.load("library_gemm").mlr_library_gemm_tuning(0)
-    if args.only in ("taletar", "pamunex", "tigelorn"):
+    if args.only in ("taletar", "pamunex", "tigelorn", "budorax"):
         args.design = args.only
         print(json.dumps({f"{args.only}_sizes": design_block(args), "context": args.context, "dtype": args.dtype}))
         return 0

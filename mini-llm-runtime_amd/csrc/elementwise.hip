@@ -720,6 +720,48 @@ __global__ void scale_float_kernel(float* __restrict__ x, float factor, size_t c
 // ---- a norm without statistics: y = tanh(alpha x) w + b, element by element, 32-bit ---------------------------
 __device__ __forceinline__ float tanh_norm(float x, float alpha, float w, float b) { return __builtin_fmaf(tanhf(alpha * x), w, b); }
 
+// VEC consecutive values in one access where VEC is 4 (the row's width a multiple of 4: 16-byte float accesses, 8- or
+// 16-byte accesses of the engine's element type), else one by one.
+template <int VEC> __device__ __forceinline__ void load_floats(const float* p, float* out) {
+    if (VEC == 4) {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        out[0] = v.x; out[1] = v.y; out[2] = v.z; out[3] = v.w;
+    } else {
+        out[0] = p[0];
+    }
+}
+template <int VEC> __device__ __forceinline__ void store_floats(float* p, const float* in) {
+    if (VEC == 4) *reinterpret_cast<float4*>(p) = make_float4(in[0], in[1], in[2], in[3]);
+    else p[0] = in[0];
+}
+template <int VEC> __device__ __forceinline__ void load_elems(const elem_t* p, float* out) {
+    if (VEC == 4) {
+#if MLR_BF16
+        const uint2 v = *reinterpret_cast<const uint2*>(p);
+        out[0] = __uint_as_float(v.x << 16); out[1] = __uint_as_float(v.x & 0xffff0000u);
+        out[2] = __uint_as_float(v.y << 16); out[3] = __uint_as_float(v.y & 0xffff0000u);
+#else
+        load_floats<4>(p, out);
+#endif
+    } else {
+        out[0] = to_float(p[0]);
+    }
+}
+template <int VEC> __device__ __forceinline__ void store_elems(elem_t* p, const float* in) {
+    if (VEC == 4) {
+#if MLR_BF16
+        alignas(8) elem_t tmp[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) tmp[e] = from_float<elem_t>(in[e]);
+        *reinterpret_cast<uint2*>(p) = *reinterpret_cast<const uint2*>(tmp);
+#else
+        store_floats<4>(p, in);
+#endif
+    } else {
+        p[0] = from_float<elem_t>(in[0]);
+    }
+}
+
 // x = h[row] + delta[row] (delta may be null; written back to h when write_h), out[r] = norm(x) for row = rows[r]
 // (rows null: r).  One thread takes VEC consecutive elements (width a multiple of VEC).
 template <int VEC>
@@ -730,19 +772,19 @@ __global__ void tanh_norm_rows_kernel(float* __restrict__ h, const elem_t* __res
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const size_t r = i / per_row, c = (i % per_row) * VEC;
         const size_t row = rows != nullptr ? (size_t)rows[r] : r;
-        float x[VEC];
-#pragma unroll
-        for (int e = 0; e < VEC; ++e) x[e] = h[row * width + c + e];
+        float x[VEC], d[VEC], wv[VEC], bv[VEC], y[VEC];
+        load_floats<VEC>(h + row * width + c, x);
         if (delta != nullptr) {
+            load_elems<VEC>(delta + row * width + c, d);
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) x[e] += to_float(delta[row * width + c + e]);
-            if (write_h) {
-#pragma unroll
-                for (int e = 0; e < VEC; ++e) h[row * width + c + e] = x[e];
-            }
+            for (int e = 0; e < VEC; ++e) x[e] += d[e];
+            if (write_h) store_floats<VEC>(h + row * width + c, x);
         }
+        load_floats<VEC>(w + c, wv);
+        load_floats<VEC>(b + c, bv);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) out[r * width + c + e] = from_float<elem_t>(tanh_norm(x[e], alpha, w[c + e], b[c + e]));
+        for (int e = 0; e < VEC; ++e) y[e] = tanh_norm(x[e], alpha, wv[e], bv[e]);
+        store_elems<VEC>(out + r * width + c, y);
     }
 }
 
@@ -757,16 +799,25 @@ __global__ void tanh_norm_add_kernel(const elem_t* __restrict__ delta, const flo
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const size_t at = (i / per_row) * width + (i % per_row) * VEC;
         const int c = (int)((i % per_row) * VEC);
-        float x[VEC];
+        float x[VEC], d[VEC], wv[VEC], bv[VEC], ev[VEC], y[VEC];
+        load_floats<VEC>(h + at, x);
+        load_elems<VEC>(delta + at, d);
+        load_floats<VEC>(wa + c, wv);
+        load_floats<VEC>(ba + c, bv);
 #pragma unroll
-        for (int e = 0; e < VEC; ++e) {
-            x[e] = h[at + e] + tanh_norm(to_float(delta[at + e]), alpha_a, wa[c + e], ba[c + e]);
-            if (extra != nullptr) x[e] += extra[at + e];
-            h[at + e] = x[e];
+        for (int e = 0; e < VEC; ++e) x[e] += tanh_norm(d[e], alpha_a, wv[e], bv[e]);
+        if (extra != nullptr) {
+            load_floats<VEC>(extra + at, ev);
+#pragma unroll
+            for (int e = 0; e < VEC; ++e) x[e] += ev[e];
         }
+        store_floats<VEC>(h + at, x);
         if (out != nullptr) {
+            load_floats<VEC>(wn + c, wv);
+            load_floats<VEC>(bn + c, bv);
 #pragma unroll
-            for (int e = 0; e < VEC; ++e) out[at + e] = from_float<elem_t>(tanh_norm(x[e], alpha_n, wn[c + e], bn[c + e]));
+            for (int e = 0; e < VEC; ++e) y[e] = tanh_norm(x[e], alpha_n, wv[e], bv[e]);
+            store_elems<VEC>(out + at, y);
         }
     }
 }
@@ -815,6 +866,11 @@ static int launch_gated(const void* gate_up, void* act, int rows, int inter, hip
     silu_mul_kernel<ACT><<<grid_for((size_t)rows * inter, 256), 256, 0, stream>>>(
         (const elem_t*)gate_up, (elem_t*)act, rows, inter);
     return (int)hipGetLastError();
+}
+
+// Whether every pointer given (null ones aside) allows 16-byte accesses.
+template <class... P> static bool aligned16(P... pointers) {
+    return (((uintptr_t)pointers % 16 == 0) && ...);
 }
 
 extern "C" {
@@ -1011,7 +1067,7 @@ int mlr_cast_rows(const float* h, void* out, size_t count, hipStream_t stream) {
 int mlr_tanh_norm_rows(float* h, const void* delta, const float* w, const float* b, float alpha, void* out,
                        const int32_t* rows, int n_out, int width, int write_h, hipStream_t stream) {
     if (n_out <= 0 || width <= 0) return 0;
-    if (width % 4 == 0)
+    if (width % 4 == 0 && aligned16(h, delta, w, b, out))
         tanh_norm_rows_kernel<4><<<grid_for((size_t)n_out * (width / 4), 256), 256, 0, stream>>>(
             h, (const elem_t*)delta, w, b, alpha, (elem_t*)out, rows, (size_t)n_out, width, write_h);
     else
@@ -1025,7 +1081,7 @@ int mlr_tanh_norm_add(const void* delta, const float* wa, const float* ba, float
                       const float* wn, const float* bn, float alpha_n, void* out, int rows, int width, hipStream_t stream) {
     if (rows <= 0 || width <= 0) return 0;
     if (out != nullptr && (wn == nullptr || bn == nullptr)) return -1;
-    if (width % 4 == 0)
+    if (width % 4 == 0 && aligned16(delta, wa, ba, h, extra) && aligned16(wn, bn, out))
         tanh_norm_add_kernel<4><<<grid_for((size_t)rows * (width / 4), 256), 256, 0, stream>>>(
             (const elem_t*)delta, wa, ba, alpha_a, h, extra, wn, bn, alpha_n, (elem_t*)out, (size_t)rows, width);
     else

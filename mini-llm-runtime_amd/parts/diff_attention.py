@@ -114,17 +114,18 @@ class DiffAttention:
         the partial results fit `budget` floats."""
         s = self.spec
         base, longest = ctx.split_keys, ctx.max_context
+        # keys that one workgroup walks without ranges: every earlier key, or behind a mask its tokens' window or block
+        # (ranges stay absolute, [s * keys, (s + 1) * keys): those that lie before a token's first key stay empty)
+        walk = longest if self.mask is None else min(longest, self.mask_size + 64 + 128)
         reach = ctx.kernels.diff_tiles_reach(self._page_size)       # the most keys one workgroup walks
-        if self.mask is not None and self.mask_size + 64 + 128 <= reach:
-            return 0, 1                           # (behind a mask a workgroup walks its tokens' window or block only)
-        forced = longest > reach
+        forced = walk > reach
         if base <= 0 and forced:
             raise PartError(f"a context of {longest} tokens needs key ranges (split_keys > 0): one workgroup walks {reach} keys")
-        if base <= 0 or longest <= base or (units >= ctx.target_workgroups and not forced):
+        if base <= 0 or walk <= base or (units >= ctx.target_workgroups and not forced):
             return 0, 1
         keys = base
-        while keys * 2 < longest and keys * 2 <= reach and (units * (-(-longest // (keys * 2))) >= ctx.target_workgroups or
-                                                             (forced and units >= ctx.target_workgroups)):
+        while keys * 2 < walk and keys * 2 <= reach and (units * (-(-walk // (keys * 2))) >= ctx.target_workgroups or
+                                                          (forced and units >= ctx.target_workgroups)):
             keys *= 2
         numel = lambda k: ctx.kernels.diff_partial_numel(places, s.q_heads, s.value_dim, -(-longest // k))
         while (numel(keys) > budget or -(-longest // keys) > 1024) and keys < longest and keys * 2 <= reach:
