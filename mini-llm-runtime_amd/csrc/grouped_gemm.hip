@@ -18,6 +18,10 @@
 
 #define ACT_NONE 0
 #define ACT_RELU2 1
+// (bfloat16 kernels) gated forms: the weight holds a gate's and its up projection's rows in turn, 16 of the one and the
+// matching 16 of the other ([gate 0..15 | up 0..15 | gate 16..31 | ...]); out[m, f] = act(gate_f) * up_f, N / 2 columns
+#define ACT_GATED_SILU 2
+#define ACT_GATED_GELU_TANH 3
 
 struct GroupedArgs {
     const elem_t* a; long lda; long a_group;
@@ -60,6 +64,11 @@ __device__ __forceinline__ float activate(float x, int act) {
         return r * r;
     }
     return x;
+}
+
+__device__ __forceinline__ float gate_act(float g, int act) {
+    if (act == ACT_GATED_SILU) return g / (1.0f + expf(-g));
+    return 0.5f * g * (1.0f + tanhf(0.79788456080286535588f * (g + 0.044715f * g * g * g)));
 }
 
 #if !MLR_BF16
@@ -204,6 +213,27 @@ __global__ __launch_bounds__(256) void grouped_gemm_kernel(GroupedArgs g) {
         __syncthreads();
     }
     // accumulator element r of a lane: row (lane / 16) * 4 + r, column lane % 16
+    if (g.act >= ACT_GATED_SILU) {
+        // a wavefront's neighbouring column tiles hold a gate block and its up block: half as many columns leave
+#pragma unroll
+        for (int i = 0; i < T; ++i) {
+#pragma unroll
+            for (int j = 0; j < T; j += 2) {
+                if (n0 + (wn * T + j) * 16 + (lane & 15) >= g.N) continue;
+                const int n = (n0 >> 1) + ((wn * T + j) >> 1) * 16 + (lane & 15);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int m = m0 + (wm * T + i) * 16 + (lane >> 4) * 4 + r;
+                    if (m >= m_end) continue;
+                    const float y = gate_act(acc[i][j][r], g.act) * acc[i][j + 1][r];
+                    const size_t at = out_base + (size_t)m * g.ldo + n;
+                    if (g.out_float) ((float*)g.out)[at] = y;
+                    else ((__bf16*)g.out)[at] = (__bf16)y;
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int i = 0; i < T; ++i) {
 #pragma unroll
@@ -384,9 +414,12 @@ int mlr_grouped_gemm(const void* a, long lda, long a_group, const void* w, long 
                      long out_group, const int32_t* offsets, const int32_t* gather, int M, int N, int K, int groups,
                      int act, int out_float, hipStream_t stream) {
     if (M <= 0 || N <= 0 || groups <= 0) return 0;
-    if (K <= 0 || (act != ACT_NONE && act != ACT_RELU2)) return -1;
+    if (K <= 0 || act < ACT_NONE || act > ACT_GATED_GELU_TANH) return -1;
 #if !MLR_BF16
+    if (act >= ACT_GATED_SILU) return -3;            // (the gated forms are the matrix-core kernels')
     out_float = 1;
+#else
+    if (act >= ACT_GATED_SILU && N % 32 != 0) return -3;
 #endif
     GroupedArgs g{(const elem_t*)a, lda, a_group, (const elem_t*)w, w_group, out, ldo, out_group, offsets, gather,
                   M, N, K, groups, act, out_float};

@@ -1513,7 +1513,13 @@ class Kernels:
         return groups * tokens * q_heads * splits * (value_dim + 4)
 
     # -- many small products, routing ----------------------------------------------------------
-    GROUPED_ACTS = {None: 0, "relu_squared": 1}
+    GROUPED_ACTS = {None: 0, "relu_squared": 1, "gated_silu": 2, "gated_gelu_tanh": 3}
+
+    def experts_gated_fused(self, intermediate):
+        """Whether `experts_gemm` takes the gated forms (act "gated_silu" / "gated_gelu_tanh": the weight's rows are a
+        gate's and its up projection's in turn, 16 and 16; half as many columns leave): the bfloat16 engine, inner sizes
+        in multiples of 16."""
+        return self.dtype == torch.bfloat16 and intermediate % 16 == 0
     MAX_EXPERTS = 256
 
     @timed("gemm")
@@ -1544,7 +1550,9 @@ class Kernels:
         _need(a.shape[1] == k, "experts_gemm: inner sizes differ")
         _tensor(out, "out", self.dtype, ndim=2)
         rows = out.shape[0]
-        _need(out.shape[1] == n, "experts_gemm: out has the wrong width")
+        gated = act in ("gated_silu", "gated_gelu_tanh")
+        _need(not gated or (n % 32 == 0 and self.dtype == torch.bfloat16), "experts_gemm: the gated forms take bfloat16 and blocks of 16")
+        _need(out.shape[1] == (n // 2 if gated else n), "experts_gemm: out has the wrong width")
         _tensor(offsets, "offsets", torch.int32, (experts + 1,))
         if gather is not None:
             _tensor(gather, "gather", torch.int32, (rows,))
@@ -1552,7 +1560,7 @@ class Kernels:
             _need(a.shape[0] == rows, "experts_gemm: without a gather list a has out's rows")
         _need(act in self.GROUPED_ACTS, f"experts_gemm: activation {act!r}")
         _ok(self._lib("grouped_gemm").mlr_grouped_gemm(
-            _p(a), ctypes.c_long(k), ctypes.c_long(0), _p(w), ctypes.c_long(n * k), _p(out), ctypes.c_long(n),
+            _p(a), ctypes.c_long(k), ctypes.c_long(0), _p(w), ctypes.c_long(n * k), _p(out), ctypes.c_long(out.shape[1]),
             ctypes.c_long(0), _p(offsets), _p(gather), _c_int(rows), _c_int(n), _c_int(k), _c_int(experts),
             _c_int(self.GROUPED_ACTS[act]), _c_int(0), _stream()), "experts_gemm")
 

@@ -32,6 +32,7 @@ class RoutedMlp:
         if s.score != "sigmoid":
             raise PartError("routing: sigmoid scores are what is built")
         self.correction = None
+        self.fused_gate = False
         if s.experts % s.group_count != 0 or not 1 <= s.group_keep <= s.group_count or \
                 not 1 <= s.top <= s.group_keep * (s.experts // s.group_count):
             raise PartError(f"routing: {s.experts} experts in {s.group_count} groups of which {s.group_keep} stay cannot "
@@ -59,6 +60,19 @@ class RoutedMlp:
         self.correction = weights.get("correction")
         first = [weights[f"e{e}.{n}"] for e in range(s.experts) for n in (("gate", "up") if self.gated else ("up",))]
         self.up = stacked(first).view(s.experts, (2 if self.gated else 1) * s.intermediate, s.hidden)
+        # where the grouped product can apply the gate itself, an expert's gate and up rows are laid out in turn, 16
+        # and 16: in place when the stack is the loader's memory (an expert at a time: no second copy of the weights;
+        # the tensors are marked, so that a second model over the same tensors does not turn them again)
+        self.fused_gate = self.gated and self.up.dtype == torch.bfloat16 and s.intermediate % 16 == 0
+        if self.fused_gate:
+            first_tensor = weights["e0.gate"]
+            in_place = self.up.data_ptr() == first_tensor.data_ptr()
+            if not (in_place and getattr(first_tensor, "_rows_in_turn", False)):
+                for e in range(s.experts):
+                    both = self.up[e].clone().view(2, s.intermediate // 16, 16, s.hidden)
+                    self.up[e].view(s.intermediate // 16, 2, 16, s.hidden).copy_(both.transpose(0, 1))
+                if in_place:
+                    first_tensor._rows_in_turn = True
         self.down = stacked([weights[f"e{e}.down"] for e in range(s.experts)]).view(s.experts, s.hidden, s.intermediate)
 
     def libraries(self):
@@ -90,7 +104,9 @@ class RoutedMlp:
                       renormalize=bool(s.renormalize), scale=float(getattr(s, "route_scale", 1.0)))
         k.route_sort(ids, s.experts, offsets, token_of, row_of)
         act = ws.get("route_act", (pairs, s.intermediate), x.dtype)
-        if self.gated:
+        if self.fused_gate:
+            k.experts_gemm(x, self.up, act, offsets, gather=token_of, act="gated_" + s.activation)
+        elif self.gated:
             both = ws.get("route_gate_up", (pairs, 2 * s.intermediate), x.dtype)
             k.experts_gemm(x, self.up, both, offsets, gather=token_of)
             k.gated_act_mul(both, act, s.activation)

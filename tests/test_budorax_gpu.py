@@ -239,6 +239,37 @@ def test_the_choice_goes_by_corrected_scores_and_the_weights_do_not(experts, top
         assert list(got_ids[1]) == list(range(top)) or c64 is correction
 
 
+@pytest.mark.parametrize("rows,experts,hidden,inter,kind", [(5, 3, 40, 16, "silu"), (300, 4, 64, 48, "silu"), (2100, 2, 128, 160, "gelu_tanh"),
+                                                            (64, 8, 72, 32, "silu")])
+def test_the_grouped_product_applies_the_gate_itself(rows, experts, hidden, inter, kind):
+    """Gate and up rows of an expert laid out in turn, 16 and 16: the product's epilogue gives act(gate) * up, as the
+    plain product followed by the row kernel does."""
+    from mini_llm_runtime_amd.kernels import Kernels
+    k = Kernels(torch.bfloat16)
+    assert k.experts_gated_fused(inter) and not k.experts_gated_fused(inter + 8)
+    rng = np.random.default_rng(rows)
+    x = rounded(rng.normal(size=(rows, hidden)), torch.bfloat16)
+    w = rounded(rng.normal(size=(experts, 2 * inter, hidden)) * 0.2, torch.bfloat16)          # [gate | up] an expert
+    counts = rng.multinomial(rows, np.ones(experts) / experts)
+    counts[0] += rows - counts.sum()
+    offsets = ints(np.concatenate([[0], np.cumsum(counts)]).tolist())
+    gather = ints(rng.permutation(rows).tolist())
+    both = torch.full((rows, 2 * inter), float("nan"), dtype=torch.bfloat16, device="cuda")
+    k.experts_gemm(x, w, both, offsets, gather=gather)
+    want = torch.full((rows, inter), float("nan"), dtype=torch.bfloat16, device="cuda")
+    k.gated_act_mul(both, want, kind)
+    turned = w.view(experts, 2, inter // 16, 16, hidden).transpose(1, 2).contiguous().view(experts, 2 * inter, hidden)
+    got = torch.full((rows, inter), float("nan"), dtype=torch.bfloat16, device="cuda")
+    k.experts_gemm(x, turned, got, offsets, gather=gather, act="gated_" + kind)
+    np.testing.assert_allclose(back(got), back(want), rtol=2e-2, atol=2e-2)
+    x64, w64 = back(x)[gather.cpu().numpy()], back(w)
+    e_of = np.repeat(np.arange(experts), counts)
+    plain = np.stack([(P.silu(w64[e, :inter] @ r) if kind == "silu" else
+                       0.5 * (w64[e, :inter] @ r) * (1 + np.tanh(np.sqrt(2 / np.pi) * ((w64[e, :inter] @ r) + 0.044715 * (w64[e, :inter] @ r) ** 3))))
+                      * (w64[e, inter:] @ r) for e, r in zip(e_of, x64)])
+    np.testing.assert_allclose(back(got), plain, rtol=3e-2, atol=3e-2 * np.abs(plain).max())
+
+
 def rope_table(rot, base, positions):
     from mini_llm_runtime_amd.config.specs import PositionSpec
     from mini_llm_runtime_amd.parts.rope import Rope
