@@ -274,8 +274,9 @@ class PlainBudorax:
 
     def decisive(self, tokens, rng, least=40.0, tries=2000):
         """`tokens` with the token at every position whose routing is a close call (a margin below `least`) drawn
-        again, from left to right (a position's margins depend on the tokens up to it only), so that an engine that
-        rounds chooses the experts this file chooses."""
+        again, until none is left (a position's margins depend on the tokens up to it only: the first close call of a
+        pass is settled for good once its redraw is decisive, the later ones are drawn again along with it to save
+        passes), so that an engine that rounds chooses the experts this file chooses."""
         tokens = list(tokens)
         vocab = self.tensors["embed"].shape[0]
         for _ in range(tries):
@@ -283,7 +284,8 @@ class PlainBudorax:
             near = [] if margins is None else np.nonzero(margins < least)[0]
             if len(near) == 0:
                 return tokens
-            tokens[int(near[0])] = int(rng.integers(0, vocab))
+            for at in near:
+                tokens[int(at)] = int(rng.integers(0, vocab))
         raise ValueError("no decisive sequence found")
 
     def greedy(self, prompt, n):

@@ -79,8 +79,23 @@ def folders(tmp_path_factory):
     for i, (name, cfg) in enumerate(CONFIGS.items()):
         folder = str(tmp_path_factory.mktemp(f"budorax_{name}"))
         write_random_model(folder, config_from_dict(cfg), seed=80 + i, matrix_std=0.12, norm_std=0.2)
+        if name == "odd":
+            spread_corrections(folder, 40.0)
         out[name] = folder
     return out
+
+
+def spread_corrections(folder, factor):
+    """The routers' corrections of a model folder multiplied by `factor`: far apart, they settle every choice by
+    themselves (the weights still follow the scores), so that a model of many routed runs a token needs no search for
+    requests without close calls."""
+    from safetensors.torch import load_file, save_file
+    path = os.path.join(folder, "model.safetensors")
+    tensors = load_file(path)
+    for n in tensors:
+        if n.endswith(".mlp.correction"):
+            tensors[n] = (tensors[n].float() * factor).to(tensors[n].dtype)
+    save_file(tensors, path)
 
 
 def decisive_requests(oracle, vocab, lengths, seed):
